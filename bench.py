@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused SAE decoder-loss path on one MI355X.
+
+One "step" = forward + backward of the HierarchicalTopK loss through the public API
+(``triton_hierarchical_sae_loss(...)``; ``loss.backward()``) on one batch of synthetic input that
+is already resident in HBM.  Default workload: B=4096, F=65536, D=2304, K=128, bf16 tensors with
+fp32 arithmetic, per-row unique uniform indices.  The TopK loss is timed on the same inputs for
+the latency ratio, the two dominant kernels are timed alone with HIP events for the roofline
+object, and a torch restatement of the reference's eager path is timed on the host cores on a
+bounded row sample as the CPU baseline.
+
+Prints ONE JSON line on stdout.  ``python bench.py --gpus 1 --steps 20 --warmup 5``.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+WORKLOADS = {
+    # name: (B, K, F, D, dtype, index distribution, weight std)
+    "c2_k128": (4096, 128, 65536, 2304, "bf16", "unique", 1.0),
+    "c2_k64": (4096, 64, 65536, 2304, "bf16", "unique", 1.0),
+    "c2_k32": (4096, 32, 65536, 2304, "bf16", "unique", 1.0),
+    "c3": (2048, 256, 131072, 1024, "fp32", "randint", 1.0),
+    "c4": (8192, 64, 262144, 4096, "bf16", "zipf", 0.02),
+    "c5": (16384, 128, 524288, 8192, "bf16", "unique", 0.02),
+    "c1": (64, 32, 4096, 256, "fp32", "randint", 1.0),
+}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2_k128", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU-baseline sample (0 = auto)")
+    return ap.parse_args()
+
+
+def make_inputs(torch, B, K, F, D, dtype, dist, w_std, device):
+    """Seeded synthetic inputs, generated on the device (indices/vals/weight/bias/target)."""
+    g = torch.Generator(device=device).manual_seed(1234)
+    if dist == "randint":
+        idx = torch.randint(0, F, (B, K), generator=g, device=device, dtype=torch.long)
+    else:
+        idx = torch.empty(B, K, dtype=torch.long, device=device)
+        step = max(1, (1 << 26) // F)
+        if dist == "zipf":
+            logp = -1.1 * torch.log(torch.arange(1, F + 1, dtype=torch.float32, device=device))
+            perm = torch.randperm(F, generator=g, device=device)
+        for b0 in range(0, B, step):
+            n = min(step, B - b0)
+            u = torch.rand(n, F, generator=g, device=device)
+            if dist == "zipf":
+                key = logp - torch.log(-torch.log(u.clamp_(1e-30, 1 - 1e-7)))
+                idx[b0:b0 + n] = perm[key.topk(K, dim=1).indices]
+            else:
+                idx[b0:b0 + n] = u.topk(K, dim=1).indices
+    vals = torch.randn(B, K, generator=g, device=device).abs()
+    if dist == "zipf":
+        vals = vals.sort(dim=1, descending=True).values
+    weight = torch.empty(F, D, dtype=dtype, device=device)
+    rows = max(1, (1 << 27) // D)
+    for f0 in range(0, F, rows):
+        n = min(rows, F - f0)
+        weight[f0:f0 + n] = (torch.randn(n, D, generator=g, device=device) * w_std).to(dtype)
+    bias = torch.randn(D, generator=g, device=device).to(dtype)
+    target = torch.randn(B, D, generator=g, device=device).to(dtype)
+    return idx, weight, vals.to(dtype), bias, target
+
+
+def algorithmic_bytes(B, K, F, D, sw, st, sv):
+    """Conservative byte model: every gathered row once per sweep, every dense output once."""
+    G = B * K * D * sw
+    T = B * D * st
+    I = B * K * (8 + sv)
+    Wb = F * D * sw
+    dv = B * K * 4
+    R = B * D * 4  # the fp32 residual handed from forward to backward
+    return {
+        "hier_step": 2 * G + 2 * T + 2 * I + Wb + dv + 8 * D,
+        "topk_step": (G + T + I) + (Wb + R + I + Wb + dv + 4 * D),
+        "fwd_kernel": G + T + I + R + D * sw,
+        "hier_bwd_kernel": G + R + I + Wb + dv + 4 * D,
+        "topk_bwd_kernel": Wb + Wb + B * K * 4 + I + dv,
+    }
+
+
+def time_steps(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def time_kernel_events(torch, prepare, launch, steps, warmup):
+    """Average duration (ms) of ``launch`` alone, HIP events on the launch stream."""
+    for _ in range(max(1, warmup)):
+        prepare()
+        launch()
+    torch.cuda.synchronize()
+    total = 0.0
+    for _ in range(steps):
+        prepare()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        launch()
+        e1.record()
+        e1.synchronize()
+        total += e0.elapsed_time(e1)
+    return total / steps
+
+
+def cpu_baseline(torch, mode_name, inputs, full_B, rows=0):
+    """The reference's eager torch path (gather -> scale -> cumsum -> MSE -> autograd) restated in
+    oracle.torch_loss, timed on the host cores on the first ``rows`` rows with the full weight
+    matrix; the per-step figure is scaled to the full batch (the work is linear in B apart from
+    the dense weight-gradient buffer, which the sample pays in full)."""
+    import oracle
+
+    # the host share of a one-GPU box is 16 cores, whatever os.cpu_count() reports there
+    threads = min(16, os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    torch.set_num_threads(threads)
+    mode = oracle.HIER if mode_name == "hier" else oracle.TOPK
+    W, b = inputs[1].cpu(), inputs[3].cpu()
+    K, D = inputs[0].shape[1], W.shape[1]
+    chunk = max(1, (1 << 28) // (K * D * 4))  # keep [Bc,K,D] fp32 around 256 MiB
+
+    def run(n):
+        idx, v, t = inputs[0][:n].cpu(), inputs[2][:n].cpu(), inputs[4][:n].cpu()
+        Wg, vg, bg = (x.detach().clone().requires_grad_() for x in (W, v, b))
+        t0 = time.perf_counter()
+        loss = oracle.torch_loss(mode, idx, Wg, vg, bg, t, chunk_rows=chunk)
+        loss.backward()
+        return time.perf_counter() - t0
+
+    if not rows:
+        probe_rows = min(full_B, 16)
+        run(probe_rows)  # warm-up (allocator, thread pool)
+        probe = run(probe_rows)
+        rows = int(min(full_B, max(probe_rows, probe_rows * 4.0 / max(probe, 1e-3))))  # ~4 s per repetition
+    else:
+        run(min(rows, full_B))
+    rows = min(rows, full_B)
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 3 and (time.perf_counter() - t_all) < 20.0:
+        times.append(run(rows))
+    sec = sum(times) / len(times)
+    return {
+        "value": round(sec * 1e3 * (full_B / rows), 1),
+        "unit": "ms",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"first {rows} of {full_B} rows with the full F x D weight, {len(times)} timed fwd+bwd "
+                  f"repetitions after a warm-up, {sec * 1e3:.1f} ms each; value = that x {full_B}/{rows}",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build measures one GPU only (the path has no multi-GPU "
+                         "code); run with --gpus 1\n")
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible\n")
+        sys.exit(3)
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import flexsae_amd as flex
+    from flexsae_amd import _lib
+
+    lib = _lib.load()  # fails loudly if the HIP library is not built
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    B, K, F, D, dt_name, dist, w_std = WORKLOADS[args.workload]
+    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[dt_name]
+    es = 2 if dtype == torch.bfloat16 else 4
+    inputs = make_inputs(torch, B, K, F, D, dtype, dist, w_std, dev)
+    idx, W, v, b, t = inputs
+    torch.cuda.synchronize()
+    abytes = algorithmic_bytes(B, K, F, D, es, es, es)
+
+    Wp, vp, bp = (x.clone().requires_grad_() for x in (W, v, b))
+
+    def step(fn):
+        Wp.grad = vp.grad = bp.grad = None
+        loss = fn(idx, Wp, vp, bp, t)
+        loss.backward()
+        return loss
+
+    torch.cuda.reset_peak_memory_stats()
+    base_mem = torch.cuda.memory_allocated()
+    hier_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
+    hier_peak = torch.cuda.max_memory_allocated() - base_mem
+    Wp.grad = vp.grad = bp.grad = None
+    torch.cuda.reset_peak_memory_stats()
+    topk_ms = time_steps(torch, lambda: step(flex.triton_topk_sae_loss), args.steps, args.warmup)
+    topk_peak = torch.cuda.max_memory_allocated() - base_mem
+    Wp.grad = vp.grad = bp.grad = None
+
+    # ---- dominant kernels alone, HIP events on the launch stream -------------------------
+    DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+    sh = _lib.Shape(B, K, F, D, DT[dtype], DT[dtype], DT[dtype], DT[dtype])
+    p = lambda x: ctypes.c_void_p(x.data_ptr())
+    st = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ws_bytes = lib.flexsae_fwd_workspace_bytes(ctypes.byref(sh))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    loss = torch.empty(1, dtype=torch.float32, device=dev)
+    resid = torch.empty(B, D, dtype=torch.float32, device=dev)
+    g1 = torch.ones(1, dtype=torch.float32, device=dev)
+    dW_acc = torch.empty(F, D, dtype=torch.float32, device=dev)
+    dvals = torch.empty(B, K, dtype=torch.float32, device=dev)
+    dbias = torch.empty(D, dtype=torch.float32, device=dev)
+
+    def fwd_launch():
+        _lib.check(lib.flexsae_hier_fwd(ctypes.byref(sh), p(idx), p(W), p(v), p(b), p(t), p(loss), p(resid), p(ws),
+                                        ws_bytes, None, st()), "flexsae_hier_fwd")
+
+    def bwd_prepare():
+        dW_acc.zero_()
+        dvals.zero_()
+        dbias.zero_()
+
+    def bwd_launch():
+        _lib.check(lib.flexsae_hier_bwd(ctypes.byref(sh), p(idx), p(W), p(v), p(resid), p(g1), p(dW_acc), p(dvals),
+                                        p(dbias), _lib.BWD_OUTPUTS_PREZEROED, None, st()), "flexsae_hier_bwd")
+
+    fwd_k_ms = time_kernel_events(torch, lambda: None, fwd_launch, args.steps, args.warmup)
+    bwd_k_ms = time_kernel_events(torch, bwd_prepare, bwd_launch, args.steps, args.warmup)
+    del dW_acc
+
+    def gbps(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9
+
+    dominant = "hier_bwd_kernel" if bwd_k_ms >= fwd_k_ms else "sae_fwd_kernel(hier)"
+    dom_bytes = abytes["hier_bwd_kernel"] if bwd_k_ms >= fwd_k_ms else abytes["fwd_kernel"]
+    dom_ms = max(bwd_k_ms, fwd_k_ms)
+    roofline = {
+        "bound": "hbm",
+        "kernel": dominant,
+        "achieved": round(gbps(dom_bytes, dom_ms), 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(gbps(dom_bytes, dom_ms) / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "algorithmic_bytes": dom_bytes,
+        "avg_launch_ms": round(dom_ms, 4),
+    }
+
+    out = {
+        "metric": "fwd+bwd ms/step + HBM GB/s (% peak), HierTopK F=65536 D=2304 K=128",
+        "value": round(hier_ms, 4),
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(hier_ms, 4),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32 arithmetic on %s storage" % dt_name,
+        "data": "synthetic",
+        "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
+                               f"indices {dist}", "B": B, "K": K, "F": F, "D": D},
+        "roofline": roofline,
+        "step_hbm": {"algorithmic_bytes": abytes["hier_step"],
+                     "achieved_GBps": round(gbps(abytes["hier_step"], hier_ms), 1),
+                     "frac_of_peak": round(gbps(abytes["hier_step"], hier_ms) / HBM_PEAK_GBPS, 4)},
+        "kernels": {
+            "sae_fwd_kernel(hier)": {"ms": round(fwd_k_ms, 4), "algorithmic_bytes": abytes["fwd_kernel"],
+                                     "GBps": round(gbps(abytes["fwd_kernel"], fwd_k_ms), 1)},
+            "hier_bwd_kernel": {"ms": round(bwd_k_ms, 4), "algorithmic_bytes": abytes["hier_bwd_kernel"],
+                                "GBps": round(gbps(abytes["hier_bwd_kernel"], bwd_k_ms), 1)},
+        },
+        "topk": {"ms_per_step": round(topk_ms, 4), "algorithmic_bytes": abytes["topk_step"],
+                 "achieved_GBps": round(gbps(abytes["topk_step"], topk_ms), 1)},
+        "hier_over_topk_latency": round(hier_ms / topk_ms, 3),
+        "peak_mem_gib": {"hier": round(hier_peak / 2 ** 30, 3), "topk": round(topk_peak / 2 ** 30, 3),
+                         "inputs": round(base_mem / 2 ** 30, 3)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, "hier", inputs, B, rows=args.cpu_rows)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

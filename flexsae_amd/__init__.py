@@ -1,0 +1,35 @@
+"""flexsae_amd: the fused SAE decoder-loss path (TopK / HierarchicalTopK, forward + backward)
+as hand-written HIP kernels for AMD MI355X (gfx950), behind the reference package's names.
+
+    import flexsae_amd as flex
+    loss = flex.triton_hierarchical_sae_loss(indices, weight, vals, bias, target)
+    loss.backward()
+
+Public names mirror reference torch-ext/flex_sae/__init__.py:5-18.  The ``triton_*`` names are
+kept so that existing callers need no edit; nothing here uses Triton.
+"""
+from .ops import (check_index_flag, set_index_checking, triton_hierarchical_sae_loss,
+                  triton_topk_sae_loss)
+from .reference import hierarchical_sae_loss, topk_sae_loss
+
+# spelled-out aliases for new code
+fused_hierarchical_sae_loss = triton_hierarchical_sae_loss
+fused_topk_sae_loss = triton_topk_sae_loss
+
+__kernel_metadata__ = {
+    "license": "Apache-2.0",
+    "backend": "hip",
+    "arch": "gfx950",
+}
+
+__all__ = [
+    "__kernel_metadata__",
+    "topk_sae_loss",
+    "triton_topk_sae_loss",
+    "hierarchical_sae_loss",
+    "triton_hierarchical_sae_loss",
+    "fused_topk_sae_loss",
+    "fused_hierarchical_sae_loss",
+    "check_index_flag",
+    "set_index_checking",
+]

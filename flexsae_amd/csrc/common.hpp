@@ -1,0 +1,163 @@
+// Device-side helpers shared by all kernels: dtype conversion, vector loads/stores,
+// wavefront (64-lane) reductions.  gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/flexsae_amd.h"
+
+namespace flexsae {
+
+constexpr int kWave = 64;
+
+// Storage tags for the 16-bit element types (the bits are handled by hand so the
+// code does not depend on any header's bf16/fp16 class).
+struct bf16_t {
+  uint16_t bits;
+};
+struct f16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
+  return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+
+// round-to-nearest-even, NaN kept quiet
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  _Float16 x;
+  __builtin_memcpy(&x, &h, 2);
+  return static_cast<float>(x);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 x = static_cast<_Float16>(f);
+  uint16_t h;
+  __builtin_memcpy(&h, &x, 2);
+  return h;
+}
+
+template <typename T>
+struct Traits;
+template <>
+struct Traits<float> {
+  using store_t = float;
+  static constexpr int dtype = FLEXSAE_F32;
+  __device__ static __forceinline__ float up(float v) { return v; }
+  __device__ static __forceinline__ float down(float v) { return v; }
+};
+template <>
+struct Traits<bf16_t> {
+  using store_t = uint16_t;
+  static constexpr int dtype = FLEXSAE_BF16;
+  __device__ static __forceinline__ float up(uint16_t v) { return bf16_bits_to_f32(v); }
+  __device__ static __forceinline__ uint16_t down(float v) { return f32_to_bf16_bits(v); }
+};
+template <>
+struct Traits<f16_t> {
+  using store_t = uint16_t;
+  static constexpr int dtype = FLEXSAE_F16;
+  __device__ static __forceinline__ float up(uint16_t v) { return f16_bits_to_f32(v); }
+  __device__ static __forceinline__ uint16_t down(float v) { return f32_to_f16_bits(v); }
+};
+
+template <typename S, int N>
+using vec_t = S __attribute__((ext_vector_type(N)));
+
+// o[0..VEC) = float(base[off .. off+VEC)); (base+off) must be aligned to VEC elements.
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec(const void *base, int64_t off, float (&o)[VEC]) {
+  using S = typename Traits<T>::store_t;
+  const S *p = static_cast<const S *>(base) + off;
+  if constexpr (VEC == 1) {
+    o[0] = Traits<T>::up(*p);
+  } else {
+    const vec_t<S, VEC> v = *reinterpret_cast<const vec_t<S, VEC> *>(p);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o[i] = Traits<T>::up(v[i]);
+  }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_vec(void *base, int64_t off, const float (&x)[VEC]) {
+  using S = typename Traits<T>::store_t;
+  S *p = static_cast<S *>(base) + off;
+  if constexpr (VEC == 1) {
+    *p = Traits<T>::down(x[0]);
+  } else {
+    vec_t<S, VEC> v;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = Traits<T>::down(x[i]);
+    *reinterpret_cast<vec_t<S, VEC> *>(p) = v;
+  }
+}
+
+// One element of a tensor whose dtype is only known at run time (vals, bias, target:
+// small tensors next to the gathered weight rows).
+__device__ __forceinline__ float load_scalar(const void *base, int dtype, int64_t i) {
+  if (dtype == FLEXSAE_F32) return static_cast<const float *>(base)[i];
+  const uint16_t h = static_cast<const uint16_t *>(base)[i];
+  return dtype == FLEXSAE_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+}
+
+// VEC consecutive elements of a run-time-typed tensor; takes the vector path when the
+// dtype equals the compile-time type T (the common case: all tensors share a dtype).
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec_dyn(const void *base, int dtype, int64_t off,
+                                             float (&o)[VEC]) {
+  if (dtype == Traits<T>::dtype) {
+    load_vec<T, VEC>(base, off, o);
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o[i] = load_scalar(base, dtype, off + i);
+  }
+}
+
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_move(float v) {
+  // lanes whose row is masked out, or whose source lane does not exist, receive 0
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+
+// Sum over the 64 lanes of the wavefront using DPP moves only (no LDS traffic).
+// The total is valid in lane 63; use wave_sum_bcast() to have it in every lane.
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+  v += dpp_move<0xB1>(v);         // quad_perm [1,0,3,2]: lane ^ 1
+  v += dpp_move<0x4E>(v);         // quad_perm [2,3,0,1]: lane ^ 2
+  v += dpp_move<0x141>(v);        // row_half_mirror: the other quad of each 8
+  v += dpp_move<0x140>(v);        // row_mirror: the other half of each 16-lane row
+  v += dpp_move<0x142, 0xa>(v);   // row_bcast15 into rows 1 and 3
+  v += dpp_move<0x143, 0xc>(v);   // row_bcast31 into rows 2 and 3
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum_bcast(float v) {
+  v = wave_sum_lane63(v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+__device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }
+
+// Wave index inside the block as a scalar (uniform) value, so that everything
+// derived from it is addressed through scalar registers.
+__device__ __forceinline__ int wave_in_block() {
+  return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+}
+
+__device__ __forceinline__ int bcast_i32(int v, int src_lane) {
+  return __builtin_amdgcn_readlane(v, src_lane);
+}
+__device__ __forceinline__ float bcast_f32(float v, int src_lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
+}
+
+}  // namespace flexsae

@@ -1,0 +1,108 @@
+// HierarchicalTopK backward: reverse sweep over K per (row, D-tile).
+#pragma once
+
+#include "common.hpp"
+
+namespace flexsae {
+
+// One wavefront per (row b, D-tile) item; a tile is 64*C columns and lane l owns the
+// columns l, l+64, ..., l+64*(C-1) of the tile.  With this interleaved ownership every
+// atomic instruction of the scatter covers 64 consecutive fp32 of one dW row (two full
+// 128-byte lines), which is the densest request the L2 atomic units can be given.
+//
+// State per lane and owned column: e = r_{b,k} - t_b (starts from the saved forward
+// residual) and S = sum_{k' >= k} scale * e_{k'}.  Walking k = K-1 .. 0:
+//   S    += scale * e                        (scale = grad_out * 2/(B*K*D))
+//   dW[idx_k]  += vals_k * S                 (fp32 atomics)
+//   dvals_k     = <W[idx_k], S>              (wave reduction; added across tiles by atomics)
+//   e    -= vals_k * W[idx_k]                (step back to r_{b,k-1} - t_b)
+// and finally dbias += S.
+template <typename WT, int C, int U>
+__global__ __launch_bounds__(256) void hier_bwd_kernel(
+    const int64_t *__restrict__ indices, const void *__restrict__ weight,
+    const void *__restrict__ vals, int vals_dtype, const float *__restrict__ resid,
+    const float *__restrict__ grad_out, float coef, float *__restrict__ dW,
+    float *__restrict__ dvals, float *__restrict__ dbias, int *status_flag, int64_t n_items,
+    int ntiles, int K, int64_t F, int D) {
+  using S_t = typename Traits<WT>::store_t;
+  const S_t *__restrict__ W = static_cast<const S_t *>(weight);
+  const int lane = lane_id();
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+  if (item >= n_items) return;  // uniform per wavefront
+  const int64_t b = item / ntiles;
+  const int tile = static_cast<int>(item - b * ntiles);
+  const int dbase = tile * (kWave * C) + lane;
+  const float scale = coef * grad_out[0];
+
+  bool act[C];
+  int dcol[C];
+  float e[C], S[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int d = dbase + c * kWave;
+    act[c] = d < D;
+    dcol[c] = act[c] ? d : 0;
+    e[c] = act[c] ? resid[b * D + d] : 0.f;
+    S[c] = 0.f;
+  }
+
+  const int64_t pair0 = b * K;
+  for (int k0 = ((K - 1) / kWave) * kWave; k0 >= 0; k0 -= kWave) {
+    const int kk = k0 + lane;
+    int64_t my_idx = 0;
+    float my_val = 0.f;
+    if (kk < K) {
+      my_idx = indices[pair0 + kk];
+      my_val = load_scalar(vals, vals_dtype, pair0 + kk);
+    }
+    if (static_cast<uint64_t>(my_idx) >= static_cast<uint64_t>(F)) {
+      if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
+      my_idx = 0;
+      my_val = 0.f;
+    }
+    const int my_row = static_cast<int>(my_idx);
+    const int n = (K - k0) < kWave ? (K - k0) : kWave;  // uniform
+    float my_dval = 0.f;
+
+    auto step = [&](int j, int64_t rowoff, const float(&w)[C]) {
+      const float v = bcast_f32(my_val, j);
+      float dot = 0.f;
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        S[c] = fmaf(scale, e[c], S[c]);
+        if (act[c]) unsafeAtomicAdd(dW + rowoff + dcol[c], S[c] * v);
+        dot = fmaf(w[c], S[c], dot);
+        e[c] = fmaf(-w[c], v, e[c]);
+      }
+      dot = wave_sum_bcast(dot);
+      if (lane == j) my_dval = dot;
+    };
+
+    int j = n - 1;
+    for (; j - (U - 1) >= 0; j -= U) {
+      float w[U][C];
+      int64_t rowoff[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        rowoff[u] = static_cast<int64_t>(bcast_i32(my_row, j - u)) * D;
+#pragma unroll
+        for (int c = 0; c < C; ++c) w[u][c] = act[c] ? Traits<WT>::up(W[rowoff[u] + dcol[c]]) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) step(j - u, rowoff[u], w[u]);
+    }
+    for (; j >= 0; --j) {
+      float w[C];
+      const int64_t rowoff = static_cast<int64_t>(bcast_i32(my_row, j)) * D;
+#pragma unroll
+      for (int c = 0; c < C; ++c) w[c] = act[c] ? Traits<WT>::up(W[rowoff + dcol[c]]) : 0.f;
+      step(j, rowoff, w);
+    }
+    if (kk < K) unsafeAtomicAdd(dvals + pair0 + kk, my_dval);
+  }
+#pragma unroll
+  for (int c = 0; c < C; ++c)
+    if (act[c]) unsafeAtomicAdd(dbias + dcol[c], S[c]);
+}
+
+}  // namespace flexsae

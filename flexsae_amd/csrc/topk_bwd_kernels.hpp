@@ -1,0 +1,305 @@
+// TopK backward: latent-major pair list (CSR) construction and the segment reduction
+// that produces dW (written once, no atomics) and dvals.
+#pragma once
+
+#include "common.hpp"
+
+namespace flexsae {
+
+// ---------------------------------------------------------------------------------
+// Pair list.  count -> exclusive scan -> fill -> sort each group ascending.
+// ---------------------------------------------------------------------------------
+
+__global__ void fill_u32_kernel(uint32_t *__restrict__ p, int64_t n, uint32_t value) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    p[i] = value;
+}
+
+// counts[f] += 1 for every pair; out-of-range indices are flagged and counted as latent 0.
+__global__ void csr_count_kernel(const int64_t *__restrict__ indices, int64_t n_pairs, int64_t F,
+                                 uint32_t *__restrict__ counts, int *status_flag) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < n_pairs;
+       p += stride) {
+    int64_t f = indices[p];
+    if (static_cast<uint64_t>(f) >= static_cast<uint64_t>(F)) {
+      if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
+      f = 0;
+    }
+    atomicAdd(counts + f, 1u);
+  }
+}
+
+// In-place exclusive scan of begin[0..F) (holding counts on entry) by a single block;
+// begin[F] receives the total and cursor[0..F) a copy of the segment starts.
+constexpr int kScanThreads = 1024;
+constexpr int kScanPerThread = 8;
+__global__ __launch_bounds__(kScanThreads) void csr_scan_kernel(uint32_t *__restrict__ begin,
+                                                                uint32_t *__restrict__ cursor,
+                                                                int64_t F) {
+  __shared__ uint32_t wave_tot[kScanThreads / kWave];
+  __shared__ uint32_t carry_s;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wv = tid >> 6;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  constexpr int64_t kChunk = static_cast<int64_t>(kScanThreads) * kScanPerThread;
+  for (int64_t base = 0; base < F; base += kChunk) {
+    uint32_t x[kScanPerThread];
+    uint32_t tsum = 0;
+    const int64_t i0 = base + static_cast<int64_t>(tid) * kScanPerThread;
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) {
+      x[i] = (i0 + i < F) ? begin[i0 + i] : 0u;
+      tsum += x[i];
+    }
+    // inclusive scan of tsum across the wavefront
+    uint32_t inc = tsum;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const uint32_t y = __shfl_up(inc, off, kWave);
+      if (lane >= off) inc += y;
+    }
+    if (lane == kWave - 1) wave_tot[wv] = inc;
+    __syncthreads();
+    uint32_t wave_off = 0;
+    for (int w = 0; w < wv; ++w) wave_off += wave_tot[w];
+    uint32_t run = carry_s + wave_off + (inc - tsum);
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) {
+      if (i0 + i < F) {
+        begin[i0 + i] = run;
+        cursor[i0 + i] = run;
+      }
+      run += x[i];
+    }
+    __syncthreads();
+    if (tid == kScanThreads - 1) carry_s = run;
+    __syncthreads();
+  }
+  if (tid == 0) begin[F] = carry_s;
+}
+
+__global__ void csr_fill_kernel(const int64_t *__restrict__ indices, int64_t n_pairs, int64_t F,
+                                uint32_t *__restrict__ cursor, uint32_t *__restrict__ map) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < n_pairs;
+       p += stride) {
+    int64_t f = indices[p];
+    if (static_cast<uint64_t>(f) >= static_cast<uint64_t>(F)) f = 0;
+    const uint32_t pos = atomicAdd(cursor + f, 1u);
+    map[pos] = static_cast<uint32_t>(p);
+  }
+}
+
+// Sort every group ascending so that the list does not depend on the order in which the
+// fill kernel's atomics happened to be served.  One wavefront per latent: groups of up to
+// 64 pairs are rank-sorted in registers (pair ids are distinct); longer ones are appended
+// to long_list for csr_sort_long_kernel.
+__global__ __launch_bounds__(256) void csr_sort_short_kernel(const uint32_t *__restrict__ begin,
+                                                             uint32_t *__restrict__ map, int64_t F,
+                                                             uint32_t *__restrict__ long_count,
+                                                             uint32_t *__restrict__ long_list) {
+  const int lane = lane_id();
+  const int64_t f = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+  if (f >= F) return;
+  const uint32_t s0 = begin[f];
+  const uint32_t n = begin[f + 1] - s0;
+  if (n <= 1) return;
+  if (n > static_cast<uint32_t>(kWave)) {
+    if (lane == 0) long_list[atomicAdd(long_count, 1u)] = static_cast<uint32_t>(f);
+    return;
+  }
+  const bool have = static_cast<uint32_t>(lane) < n;
+  const uint32_t x = have ? map[s0 + lane] : 0xffffffffu;
+  uint32_t rank = 0;
+  for (uint32_t j = 0; j < n; ++j) {
+    const uint32_t y = static_cast<uint32_t>(bcast_i32(static_cast<int>(x), static_cast<int>(j)));
+    rank += (y < x) ? 1u : 0u;
+  }
+  if (have) map[s0 + rank] = x;  // every lane read its element before any lane writes
+}
+
+// Long groups: in-place bitonic network in which every comparator points the same way
+// (first sub-step of each merge mirrors, the rest are plain strides), so a length that is
+// not a power of two is handled by skipping comparators whose partner lies beyond the end.
+__global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
+                                                            uint32_t *__restrict__ map,
+                                                            const uint32_t *__restrict__ long_count,
+                                                            const uint32_t *__restrict__ long_list) {
+  const uint32_t n_long = *long_count;
+  for (uint32_t w = blockIdx.x; w < n_long; w += gridDim.x) {
+    const uint32_t f = long_list[w];
+    uint32_t *a = map + begin[f];
+    const uint32_t n = begin[f + 1] - begin[f];
+    uint32_t np2 = 1;
+    while (np2 < n) np2 <<= 1;
+    for (uint32_t k = 2; k <= np2; k <<= 1) {
+      // mirrored sub-step: inside each block of k, position i pairs with (k-1-i)
+      for (uint32_t t = threadIdx.x; t < np2 / 2; t += blockDim.x) {
+        const uint32_t blk = t / (k / 2), i = t % (k / 2);
+        const uint32_t lo = blk * k + i, hi = blk * k + (k - 1 - i);
+        if (hi < n) {
+          const uint32_t x = a[lo], y = a[hi];
+          if (x > y) {
+            a[lo] = y;
+            a[hi] = x;
+          }
+        }
+      }
+      __syncthreads();
+      for (uint32_t j = k / 4; j > 0; j >>= 1) {
+        for (uint32_t t = threadIdx.x; t < np2 / 2; t += blockDim.x) {
+          const uint32_t lo = (t / j) * (2 * j) + (t % j), hi = lo + j;
+          if (hi < n) {
+            const uint32_t x = a[lo], y = a[hi];
+            if (x > y) {
+              a[lo] = y;
+              a[hi] = x;
+            }
+          }
+        }
+        __syncthreads();
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Segment reduction.
+// ---------------------------------------------------------------------------------
+
+// One wavefront per (latent f, D-tile) item, tile = 64*VEC columns, lane l owning VEC
+// consecutive columns.  For every pair p=(b,t) of the latent's group:
+//   dW[f]    += vals[p] * g_b          g_b = scale * resid[b]   (scale = grad_out * 2/(B*D))
+//   dvals[p] += <g_b, W[f]>            (one wave reduction per pair and tile, then an atomic)
+// dW[f, tile] is written exactly once, in the gradient's final dtype; latents without pairs
+// get zeros.  resid rows are read through the caches (the [B,D] matrix is small next to W).
+// TILE_MAJOR orders the items tile by tile, so that at any moment the waves in flight share
+// one B x tile slice of resid.
+template <typename WT, typename GT, int VEC, int U, bool TILE_MAJOR>
+__global__ __launch_bounds__(256) void topk_bwd_kernel(
+    const uint32_t *__restrict__ begin, const uint32_t *__restrict__ map,
+    const void *__restrict__ weight, const void *__restrict__ vals, int vals_dtype,
+    const float *__restrict__ resid, const float *__restrict__ grad_out, float coef,
+    void *__restrict__ dW, float *__restrict__ dvals, int64_t n_items, int ntiles, int64_t F,
+    int K, int D) {
+  const int lane = lane_id();
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+  if (item >= n_items) return;  // uniform per wavefront
+  int64_t f;
+  int tile;
+  if constexpr (TILE_MAJOR) {
+    tile = static_cast<int>(item / F);
+    f = item - static_cast<int64_t>(tile) * F;
+  } else {
+    f = item / ntiles;
+    tile = static_cast<int>(item - f * ntiles);
+  }
+  const int d0 = tile * (kWave * VEC) + lane * VEC;
+  const bool active = d0 < D;
+  const int dsafe = active ? d0 : 0;
+  const float scale = coef * grad_out[0];
+
+  float w[VEC], acc[VEC];
+  load_vec<WT, VEC>(weight, f * D + dsafe, w);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    acc[i] = 0.f;
+    if (!active) w[i] = 0.f;
+  }
+
+  const uint32_t s_begin = begin[f];
+  const uint32_t s_end = begin[f + 1];
+  for (uint32_t s = s_begin; s < s_end; s += kWave) {
+    const uint32_t slot = s + lane;
+    uint32_t p = 0;
+    float v = 0.f;
+    if (slot < s_end) {
+      p = map[slot];
+      v = load_scalar(vals, vals_dtype, p) * scale;
+    }
+    const int my_b = static_cast<int>(p / static_cast<uint32_t>(K));
+    const int n = (s_end - s) < static_cast<uint32_t>(kWave) ? static_cast<int>(s_end - s) : kWave;
+    float my_dot = 0.f;
+
+    auto step = [&](int j, const float(&g)[VEC]) {
+      const float vj = bcast_f32(v, j);
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        acc[i] = fmaf(vj, g[i], acc[i]);
+        dot = fmaf(g[i], w[i], dot);
+      }
+      dot = wave_sum_bcast(dot);
+      if (lane == j) my_dot = dot;
+    };
+
+    int j = 0;
+    for (; j + U <= n; j += U) {
+      float g[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t brow = bcast_i32(my_b, j + u);
+        load_vec<float, VEC>(resid, brow * D + dsafe, g[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) step(j + u, g[u]);
+    }
+    for (; j < n; ++j) {
+      float g[VEC];
+      const int64_t brow = bcast_i32(my_b, j);
+      load_vec<float, VEC>(resid, brow * D + dsafe, g);
+      step(j, g);
+    }
+    if (slot < s_end) unsafeAtomicAdd(dvals + p, my_dot * scale);
+  }
+  if (active) store_vec<GT, VEC>(dW, f * D + d0, acc);
+}
+
+// dbias[d] += scale * sum_b resid[b, d]: grid (column blocks, row chunks).
+__global__ __launch_bounds__(256) void colsum_kernel(const float *__restrict__ resid,
+                                                     const float *__restrict__ grad_out, float coef,
+                                                     float *__restrict__ dbias, int64_t B, int D,
+                                                     int rows_per_block) {
+  const int d = blockIdx.x * blockDim.x + threadIdx.x;
+  if (d >= D) return;
+  const int64_t b0 = static_cast<int64_t>(blockIdx.y) * rows_per_block;
+  const int64_t b1 = (b0 + rows_per_block) < B ? (b0 + rows_per_block) : B;
+  float s = 0.f;
+  for (int64_t b = b0; b < b1; ++b) s += resid[b * D + d];
+  unsafeAtomicAdd(dbias + d, s * coef * grad_out[0]);
+}
+
+__global__ void fill_f32_kernel(float *__restrict__ p, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t n4 = n >> 2;
+  float4 *p4 = reinterpret_cast<float4 *>(p);
+  const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride)
+    p4[i] = z;
+  for (int64_t i = (n4 << 2) + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += stride)
+    p[i] = 0.f;
+}
+
+template <typename GT>
+__global__ void cast_from_f32_kernel(void *__restrict__ dst, const float *__restrict__ src,
+                                     int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t n4 = n >> 2;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    float x[4];
+    load_vec<float, 4>(src, i * 4, x);
+    store_vec<GT, 4>(dst, i * 4, x);
+  }
+  for (int64_t i = (n4 << 2) + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    float x[1] = {src[i]};
+    store_vec<GT, 1>(dst, i, x);
+  }
+}
+
+}  // namespace flexsae

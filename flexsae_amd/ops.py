@@ -1,0 +1,274 @@
+"""torch.library custom ops over the C-ABI HIP library, with autograd and fake (meta) kernels.
+
+Op graph (names under the ``flexsae_amd::`` namespace):
+
+    hier_fwd(indices, weight, vals, bias, target) -> (loss, resid)
+    hier_bwd(grad_out, indices, weight, vals, resid) -> (dW, dvals, dbias)
+    topk_fwd(indices, weight, vals, bias, target) -> (loss, resid)
+    topk_bwd(grad_out, indices, weight, vals, resid) -> (dW, dvals, dbias)
+
+``resid[B,D]`` (fp32) is the reconstruction error of the full row, the only state kept between
+forward and backward.  The ops take the place of the reference's two ``autograd.Function``
+classes (reference torch-ext/flex_sae/hierarchical_kernels.py:273-299 and
+torch-ext/flex_sae/topk_kernels.py:188-223) and keep their contract: gradients for ``weight``,
+``vals`` and ``bias`` only (plus ``target`` for TopK, whose loss tail is differentiable there),
+``indices`` never, an arbitrary scalar upstream gradient, no autocast of the inputs.
+
+Everything runs on the current stream of the tensors' device; nothing synchronises unless
+index checking is switched on.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+
+# device index -> int32[1] status flag the kernels OR error bits into (never reset by the ops)
+_status_flags = {}
+_check_indices = os.environ.get("FLEXSAE_CHECK_INDICES", "0") not in ("", "0")
+
+
+def set_index_checking(enabled: bool) -> None:
+    """When enabled every fused call synchronises and raises on an out-of-range index.
+
+    Off by default (the reference never checks; here such an index is neutralised on the
+    device -- treated as latent 0 with value 0 -- and recorded in a flag instead of reading
+    out of bounds)."""
+    global _check_indices
+    _check_indices = bool(enabled)
+
+
+def _flag_for(device: torch.device) -> Tensor:
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    flag = _status_flags.get(key)
+    if flag is None:
+        flag = torch.zeros(1, dtype=torch.int32, device=device)
+        _status_flags[key] = flag
+    return flag
+
+
+def check_index_flag(device=None) -> None:
+    """Synchronise and raise IndexError if any fused call since the last check saw an index
+    outside ``[0, F)``; clears the flag."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    flag = _flag_for(dev)
+    bits = int(flag.item())
+    if bits:
+        flag.zero_()
+        if bits & _lib.FLAG_INDEX_RANGE:
+            raise IndexError("flexsae_amd: an entry of `indices` was outside [0, F)")
+        raise RuntimeError(f"flexsae_amd: device status flag {bits:#x}")
+
+
+def _validate(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, target: Tensor):
+    """Shape/dtype/device checks the reference leaves to undefined behaviour."""
+    if indices.dim() != 2 or weight.dim() != 2 or vals.dim() != 2 or bias.dim() != 1 or target.dim() != 2:
+        raise ValueError("expected indices[B,K], weight[F,D], vals[B,K], bias[D], target[B,D]")
+    B, K = indices.shape
+    F, D = weight.shape
+    if tuple(vals.shape) != (B, K) or tuple(bias.shape) != (D,) or tuple(target.shape) != (B, D):
+        raise ValueError(
+            f"shape mismatch: indices{tuple(indices.shape)} weight{tuple(weight.shape)} "
+            f"vals{tuple(vals.shape)} bias{tuple(bias.shape)} target{tuple(target.shape)}")
+    if B == 0 or K == 0 or F == 0 or D == 0:
+        raise ValueError("empty inputs are not supported (B, K, F, D must all be >= 1)")
+    if indices.dtype != torch.int64:
+        raise TypeError(f"indices must be int64, got {indices.dtype}")
+    for name, t in (("weight", weight), ("vals", vals), ("bias", bias), ("target", target)):
+        if t.dtype not in _DTYPES:
+            raise TypeError(f"{name} must be float32, bfloat16 or float16, got {t.dtype}")
+    dev = weight.device
+    if dev.type != "cuda":
+        raise RuntimeError(
+            "flexsae_amd fused ops run on an AMD GPU only (tensors must live on a 'cuda' device); "
+            "use flexsae_amd.topk_sae_loss / hierarchical_sae_loss for the eager torch definition")
+    for name, t in (("indices", indices), ("vals", vals), ("bias", bias), ("target", target)):
+        if t.device != dev:
+            raise RuntimeError(f"{name} is on {t.device}, weight on {dev}")
+    if B * K >= 2 ** 32 or F >= 2 ** 31 or D >= 2 ** 31:
+        raise ValueError("sizes beyond the kernels' index range: need B*K < 2^32, F < 2^31, D < 2^31")
+    return B, K, F, D
+
+
+def _shape(B, K, F, D, weight: Tensor, vals: Tensor, bias_dtype, target_dtype) -> _lib.Shape:
+    return _lib.Shape(B, K, F, D, _DTYPES[weight.dtype], _DTYPES[vals.dtype], _DTYPES[bias_dtype],
+                      _DTYPES[target_dtype])
+
+
+def _ptr(t: Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _forward(entry: str, indices, weight, vals, bias, target) -> Tuple[Tensor, Tensor]:
+    B, K, F, D = _validate(indices, weight, vals, bias, target)
+    lib = _lib.load()
+    indices, weight, vals, bias, target = (t.contiguous() for t in (indices, weight, vals, bias, target))
+    dev = weight.device
+    with torch.cuda.device(dev):
+        shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
+        ws_bytes = lib.flexsae_fwd_workspace_bytes(ctypes.byref(shape))
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        resid = torch.empty((B, D), dtype=torch.float32, device=dev)
+        flag = _flag_for(dev)
+        rc = getattr(lib, entry)(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
+                                 _ptr(target), _ptr(loss), _ptr(resid), _ptr(workspace), ws_bytes,
+                                 _ptr(flag), _stream())
+        _lib.check(rc, entry)
+        if _check_indices:
+            check_index_flag(dev)
+    return loss, resid
+
+
+def _grad_scalar(grad_out: Tensor, dev) -> Tensor:
+    return grad_out.detach().to(device=dev, dtype=torch.float32).reshape(1).contiguous()
+
+
+@torch.library.custom_op("flexsae_amd::hier_fwd", mutates_args=())
+def hier_fwd(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
+             target: Tensor) -> Tuple[Tensor, Tensor]:
+    return _forward("flexsae_hier_fwd", indices, weight, vals, bias, target)
+
+
+@torch.library.custom_op("flexsae_amd::topk_fwd", mutates_args=())
+def topk_fwd(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
+             target: Tensor) -> Tuple[Tensor, Tensor]:
+    return _forward("flexsae_topk_fwd", indices, weight, vals, bias, target)
+
+
+def _fwd_fake(indices, weight, vals, bias, target):
+    B, _ = indices.shape
+    D = weight.shape[1]
+    return (weight.new_empty((), dtype=torch.float32), weight.new_empty((B, D), dtype=torch.float32))
+
+
+hier_fwd.register_fake(_fwd_fake)
+topk_fwd.register_fake(_fwd_fake)
+
+
+@torch.library.custom_op("flexsae_amd::hier_bwd", mutates_args=())
+def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
+             resid: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+    lib = _lib.load()
+    B, K = indices.shape
+    F, D = weight.shape
+    dev = weight.device
+    indices, weight, vals, resid = (t.contiguous() for t in (indices, weight, vals, resid))
+    with torch.cuda.device(dev):
+        g = _grad_scalar(grad_out, dev)
+        shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
+        dW_acc = torch.empty((F, D), dtype=torch.float32, device=dev)
+        dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
+        dbias = torch.empty((D,), dtype=torch.float32, device=dev)
+        rc = lib.flexsae_hier_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(resid),
+                                  _ptr(g), _ptr(dW_acc), _ptr(dvals), _ptr(dbias), 0,
+                                  _ptr(_flag_for(dev)), _stream())
+        _lib.check(rc, "flexsae_hier_bwd")
+        if weight.dtype == torch.float32:
+            dW = dW_acc
+        else:
+            dW = torch.empty_like(weight)
+            rc = lib.flexsae_cast_from_f32(_ptr(dW), _DTYPES[weight.dtype], _ptr(dW_acc), F * D, _stream())
+            _lib.check(rc, "flexsae_cast_from_f32")
+    return dW, dvals, dbias
+
+
+@torch.library.custom_op("flexsae_amd::topk_bwd", mutates_args=())
+def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
+             resid: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+    lib = _lib.load()
+    B, K = indices.shape
+    F, D = weight.shape
+    dev = weight.device
+    indices, weight, vals, resid = (t.contiguous() for t in (indices, weight, vals, resid))
+    with torch.cuda.device(dev):
+        g = _grad_scalar(grad_out, dev)
+        shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
+        begin = torch.empty(F + 1, dtype=torch.int32, device=dev)   # uint32 payload
+        pair_map = torch.empty(B * K, dtype=torch.int32, device=dev)  # uint32 payload
+        ws_bytes = lib.flexsae_csr_workspace_bytes(B, K, F)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        rc = lib.flexsae_csr_build(_ptr(indices), B, K, F, _ptr(begin), _ptr(pair_map), _ptr(workspace),
+                                   ws_bytes, _ptr(_flag_for(dev)), _stream())
+        _lib.check(rc, "flexsae_csr_build")
+        dW = torch.empty_like(weight)
+        dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
+        dbias = torch.empty((D,), dtype=torch.float32, device=dev)
+        rc = lib.flexsae_topk_bwd(ctypes.byref(shape), _ptr(begin), _ptr(pair_map), _ptr(weight), _ptr(vals),
+                                  _ptr(resid), _ptr(g), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals),
+                                  _ptr(dbias), 0, _stream())
+        _lib.check(rc, "flexsae_topk_bwd")
+    return dW, dvals, dbias
+
+
+def _bwd_fake(grad_out, indices, weight, vals, resid):
+    return (torch.empty_like(weight), vals.new_empty(vals.shape, dtype=torch.float32),
+            weight.new_empty((weight.shape[1],), dtype=torch.float32))
+
+
+hier_bwd.register_fake(_bwd_fake)
+topk_bwd.register_fake(_bwd_fake)
+
+
+def _setup_context(ctx, inputs, output):
+    indices, weight, vals, bias, target = inputs
+    _, resid = output
+    ctx.save_for_backward(indices, weight, vals, resid)
+    ctx.leaf_dtypes = (vals.dtype, bias.dtype, target.dtype)
+
+
+def _hier_backward(ctx, grad_loss, grad_resid):
+    indices, weight, vals, resid = ctx.saved_tensors
+    if grad_loss is None:
+        return None, None, None, None, None
+    dW, dvals, dbias = hier_bwd(grad_loss, indices, weight, vals, resid)
+    vdt, bdt, _ = ctx.leaf_dtypes
+    # no gradient for target on this path (reference hierarchical_kernels.py:299)
+    return None, dW, dvals.to(vdt), dbias.to(bdt), None
+
+
+def _topk_backward(ctx, grad_loss, grad_resid):
+    indices, weight, vals, resid = ctx.saved_tensors
+    if grad_loss is None:
+        return None, None, None, None, None
+    dW, dvals, dbias = topk_bwd(grad_loss, indices, weight, vals, resid)
+    vdt, bdt, tdt = ctx.leaf_dtypes
+    dtarget = None
+    if ctx.needs_input_grad[4]:
+        # the reference's eager loss tail is differentiable w.r.t. target (topk_kernels.py:221)
+        B, D = resid.shape
+        dtarget = (resid * (grad_loss.to(torch.float32) * (-2.0 / (B * D)))).to(tdt)
+    return None, dW, dvals.to(vdt), dbias.to(bdt), dtarget
+
+
+hier_fwd.register_autograd(_hier_backward, setup_context=_setup_context)
+topk_fwd.register_autograd(_topk_backward, setup_context=_setup_context)
+
+
+def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
+                                 target: Tensor) -> Tensor:
+    """Fused HierarchicalTopK decoder loss (0-dim fp32), differentiable w.r.t. weight, vals, bias.
+
+    Same name, argument order and meaning as the reference entry point
+    (torch-ext/flex_sae/hierarchical_kernels.py:302-309); the kernels underneath are HIP."""
+    return hier_fwd(indices, weight, vals, bias, target)[0]
+
+
+def triton_topk_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
+                         target: Tensor) -> Tensor:
+    """Fused TopK decoder loss (0-dim fp32), differentiable w.r.t. weight, vals, bias, target.
+
+    Same name, argument order and meaning as the reference entry point
+    (torch-ext/flex_sae/topk_kernels.py:213-223); the kernels underneath are HIP."""
+    return topk_fwd(indices, weight, vals, bias, target)[0]

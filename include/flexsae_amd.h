@@ -1,0 +1,149 @@
+/*
+ * flexsae_amd -- C ABI of the MI355X (gfx950) implementation of the fused SAE
+ * decoder-loss path: TopK and HierarchicalTopK loss, forward and backward.
+ *
+ * Every entry point takes raw device pointers and sizes, launches its kernels on
+ * the given HIP stream and returns immediately (no allocation, no
+ * synchronisation, no host<->device copy, no global state).  Return value:
+ * FLEXSAE_OK or a negative flexsae_status; nothing throws or aborts.
+ *
+ * Conventions shared by all entry points
+ *   - Tensors are contiguous row-major: indices[B,K] int64, weight[F,D],
+ *     vals[B,K], bias[D], target[B,D]; weight/vals/bias/target each carry their
+ *     own flexsae_dtype (fp32, bf16 or fp16) and are upcast to fp32 on load; all
+ *     arithmetic and accumulation is fp32.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *   - `status_flag` (may be NULL) is a device int that kernels OR bits into:
+ *     FLEXSAE_FLAG_INDEX_RANGE when an index lies outside [0,F).  Such an index
+ *     is treated as latent 0 with value 0 so that no kernel ever reads or writes
+ *     outside the tensors; the caller decides when to look at the flag.
+ *   - `grad_out` is a DEVICE pointer to the upstream fp32 scalar gradient; it is
+ *     folded into the kernels' scale factor, so there is no separate pass that
+ *     multiplies the gradients afterwards.
+ *   - Workspaces must be 256-byte aligned; their contents need not be
+ *     initialised and are garbage afterwards.
+ *
+ * "replaces" comments name the reference function (file:line under the reference
+ * checkout, torch-ext/flex_sae/) whose work the entry point takes over.
+ */
+#ifndef FLEXSAE_AMD_H
+#define FLEXSAE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLEXSAE_ABI_VERSION 1
+
+typedef enum {
+  FLEXSAE_OK = 0,
+  FLEXSAE_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive size, bad enum      */
+  FLEXSAE_ERR_UNSUPPORTED = -2,      /* size beyond what the kernels index (see below) */
+  FLEXSAE_ERR_WORKSPACE = -3,        /* workspace missing, too small or misaligned     */
+  FLEXSAE_ERR_LAUNCH = -4,           /* the HIP runtime refused a launch               */
+  FLEXSAE_ERR_ALIGNMENT = -5         /* a tensor pointer is not aligned to its element */
+} flexsae_status;
+
+typedef enum { FLEXSAE_F32 = 0, FLEXSAE_BF16 = 1, FLEXSAE_F16 = 2 } flexsae_dtype;
+
+enum { FLEXSAE_FLAG_INDEX_RANGE = 1 };
+
+/* flags for the backward entry points */
+enum {
+  FLEXSAE_BWD_OUTPUTS_PREZEROED = 1 /* caller already zero-filled the accumulators */
+};
+
+/* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^31; B*K < 2^32. */
+typedef struct {
+  int64_t B, K, F, D;
+  int32_t weight_dtype, vals_dtype, bias_dtype, target_dtype; /* flexsae_dtype */
+} flexsae_shape;
+
+int flexsae_abi_version(void);
+const char *flexsae_status_string(int status);
+
+/* Bytes of workspace the two forward entry points need for `shape`. */
+size_t flexsae_fwd_workspace_bytes(const flexsae_shape *shape);
+
+/*
+ * HierarchicalTopK forward.
+ * replaces: _hierarchical_sae_forward + hierarchical_sae_forward_kernel and the
+ *           host-side loss_per_batch.sum()/(B*K*D)  (hierarchical_kernels.py:12-89, 190-227)
+ * out: loss[1] fp32 (mean over B*K*D of (r_{b,k,d}-t_{b,d})^2, summed in a fixed order);
+ *      resid[B,D] fp32 = r_{b,K-1} - target_b, the only state the backward needs
+ *      (the reference saves final_recon and re-reads target instead).
+ */
+int flexsae_hier_fwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
+                     const void *vals, const void *bias, const void *target, float *loss,
+                     float *resid, void *workspace, size_t workspace_bytes, int *status_flag,
+                     void *stream);
+
+/*
+ * TopK forward, fully fused (gather, scale, sum over K, + bias, - target, mean square).
+ * replaces: embedding_bag_forward + embedding_bag_forward_kernel and the eager tail
+ *           of triton_topk_sae_loss  (topk_kernels.py:15-68, 213-223)
+ * out: loss[1] fp32 (mean over B*D); resid[B,D] fp32 = r_b - target_b.
+ */
+int flexsae_topk_fwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
+                     const void *vals, const void *bias, const void *target, float *loss,
+                     float *resid, void *workspace, size_t workspace_bytes, int *status_flag,
+                     void *stream);
+
+/*
+ * HierarchicalTopK backward: reverse sweep over K per row.
+ * replaces: _hierarchical_sae_backward + hierarchical_sae_backward_kernel and the three
+ *           mul_(grad) passes of HierarchicalSAELossFunction.backward
+ *           (hierarchical_kernels.py:92-187, 230-270, 294-297)
+ * in : resid from flexsae_hier_fwd; grad_out device scalar.
+ * out: dW_acc[F,D] fp32 (scatter-add accumulator), dvals[B,K] fp32, dbias[D] fp32, all
+ *      zero-filled here unless FLEXSAE_BWD_OUTPUTS_PREZEROED is set in `flags`.
+ */
+int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
+                     const void *vals, const float *resid, const float *grad_out, float *dW_acc,
+                     float *dvals, float *dbias, int flags, int *status_flag, void *stream);
+
+/* Bytes of workspace flexsae_csr_build needs. */
+size_t flexsae_csr_workspace_bytes(int64_t B, int64_t K, int64_t F);
+
+/*
+ * Latent-major pair list for the TopK backward: begin[F+1] (exclusive prefix of
+ * the per-latent pair counts, begin[F] = B*K) and map[B*K] holding pair ids
+ * p = b*K + t grouped by latent, ascending inside a group (a stable counting
+ * sort, so the result is deterministic).
+ * replaces: count_per_embedding_kernel, count.cumsum(0), map_embeddings_and_outputs_kernel
+ *           (topk_kernels.py:71-94, 149-163; there the order inside a group is racy)
+ */
+int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, uint32_t *begin,
+                      uint32_t *map, void *workspace, size_t workspace_bytes, int *status_flag,
+                      void *stream);
+
+/*
+ * TopK backward: latent-major segment reduction (no atomics on dW).
+ * replaces: aggregate_gradient_for_embedding_kernel and its launch, plus the autograd of
+ *           the eager loss tail that produces `gradient` and the bias gradient
+ *           (topk_kernels.py:97-137, 165-184, 220-223)
+ * in : begin/map from flexsae_csr_build; resid from flexsae_topk_fwd; grad_out device scalar.
+ * out: dW[F,D] written once in `dW_dtype` (every row, zeros for unused latents);
+ *      dvals[B,K] fp32 and dbias[D] fp32 (zero-filled here unless
+ *      FLEXSAE_BWD_OUTPUTS_PREZEROED).
+ */
+int flexsae_topk_bwd(const flexsae_shape *shape, const uint32_t *begin, const uint32_t *map,
+                     const void *weight, const void *vals, const float *resid,
+                     const float *grad_out, void *dW, int dW_dtype, float *dvals, float *dbias,
+                     int flags, void *stream);
+
+/*
+ * dst[n] (dtype) = src[n] (fp32), round-to-nearest-even.  Used to hand the fp32
+ * scatter accumulator of the hierarchical backward over in the weight's dtype.
+ * replaces: the autograd engine's implicit cast of the fp32 gradients returned at
+ *           hierarchical_kernels.py:299.
+ */
+int flexsae_cast_from_f32(void *dst, int dst_dtype, const float *src, int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLEXSAE_AMD_H */

@@ -1,0 +1,272 @@
+"""GPU parity tests: HIP kernels (through the C-ABI and through the torch ops) vs the CPU oracle.
+
+Tolerances (normwise relative error, ||got-ref|| / ||ref||):
+  fp32 : 1e-5 on the loss, 1e-4 on dvals / dW / dbias
+  bf16 : 1e-2 on everything;  fp16 : 1e-3
+and, on the reference's own shape x dtype matrix, also torch.testing.assert_close with the
+reference's per-dtype atol/rtol (reference tests/test_setup.py:35-39).  Integer outputs (the
+latent-major pair list) and gather addressing are compared bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+import abi
+import flexsae_amd as flex
+import oracle
+from helpers import DTYPE_TO_TOLS, PARAMS, REL_TOL, make_inputs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+MODES = {"hier": oracle.HIER, "topk": oracle.TOPK}
+FUSED = {"hier": flex.triton_hierarchical_sae_loss, "topk": flex.triton_topk_sae_loss}
+
+
+def _to_dev(args):
+    return [a.to(DEV) for a in args]
+
+
+def _announce(*what):
+    print("[case]", *what, flush=True)
+
+
+def _run_op(mode, args_cpu, grad_out):
+    idx, W, v, b, t = _to_dev(args_cpu)
+    W.requires_grad_()
+    v.requires_grad_()
+    b.requires_grad_()
+    loss = FUSED[mode](idx, W, v, b, t)
+    loss.backward(torch.tensor(grad_out, device=DEV, dtype=torch.float32))
+    torch.cuda.synchronize()
+    assert idx.grad is None and t.grad is None
+    return loss, W.grad, v.grad, b.grad
+
+
+def _check_against_oracle(mode, args_cpu, dtype, grad_out, got, ref_tols=True):
+    loss, dW, dv, db = got
+    L, rW, rv, rb = oracle.loss_grads(MODES[mode], *args_cpu, grad_out=grad_out)
+    tol_loss, tol_grad = REL_TOL[dtype]
+    assert loss.dtype == torch.float32 and loss.dim() == 0
+    assert abs(loss.item() - L) <= tol_loss * abs(L), (loss.item(), L)
+    assert dW.dtype == dtype and dv.dtype == dtype and db.dtype == dtype
+    for name, g, r in (("dW", dW, rW), ("dvals", dv, rv), ("dbias", db, rb)):
+        err = rel_err(g.float().cpu(), r)
+        assert err <= tol_grad, f"{name}: rel err {err:.3e} > {tol_grad}"
+    if ref_tols:
+        tols = DTYPE_TO_TOLS[dtype]
+        torch.testing.assert_close(loss.cpu(), torch.tensor(L, dtype=torch.float32), **tols)
+        for g, r in ((dW, rW), (dv, rv), (db, rb)):
+            torch.testing.assert_close(g.cpu(), torch.from_numpy(r).to(dtype), **tols)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("B,K,F,D", PARAMS)
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_reference_matrix(mode, B, K, F, D, dtype):
+    """The reference's 26 shapes x 3 dtypes x 2 losses, with a random scalar upstream gradient
+    (reference tests/test_all_kernels.py:20-66)."""
+    _announce("matrix", mode, B, K, F, D, dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype)
+    grad_out = float(torch.randn((), generator=torch.Generator().manual_seed(B * K + D)))
+    got = _run_op(mode, args, grad_out)
+    _check_against_oracle(mode, args, dtype, grad_out, got)
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (3, 5, 7, 9), (5, 3, 11, 70), (2, 65, 40, 130),
+                                   (7, 130, 300, 200), (4, 24, 50, 1000), (33, 12, 17, 2304)])
+def test_odd_shapes_fp32(mode, shape):
+    """Sizes the reference's static asserts reject: K not a power of two, K > 64 with a ragged
+    last group, D not a multiple of 64 (nor of the vector width), B not a multiple of 16."""
+    B, K, F, D = shape
+    _announce("odd", mode, shape)
+    args = make_inputs(B, K, F, D, seed=B + K + F + D)
+    got = _run_op(mode, args, -1.25)
+    _check_against_oracle(mode, args, torch.float32, -1.25, got, ref_tols=False)
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_mixed_dtypes(mode):
+    """weight/vals/bias/target each in a different dtype (the reference upcasts each load on its
+    own: hierarchical_kernels.py:49-64, topk_kernels.py:38)."""
+    _announce("mixed", mode)
+    idx, W, v, b, t = make_inputs(24, 16, 90, 384, seed=21)
+    args = (idx, W.to(torch.bfloat16), v.to(torch.float16), b.to(torch.float32), t.to(torch.float16))
+    loss, dW, dv, db = _run_op(mode, args, 0.5)
+    L, rW, rv, rb = oracle.loss_grads(MODES[mode], *args, grad_out=0.5)
+    assert abs(loss.item() - L) <= 1e-5 * abs(L)
+    assert (dW.dtype, dv.dtype, db.dtype) == (torch.bfloat16, torch.float16, torch.float32)
+    assert rel_err(dW.float().cpu(), rW) < 1e-2
+    assert rel_err(dv.float().cpu(), rv) < 1e-3
+    assert rel_err(db.cpu(), rb) < 1e-4
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_gather_addressing_is_exact(mode, dtype):
+    """Identity-style weight: W[f,d] holds an integer code of (f,d), vals = 1, bias = target = 0,
+    so resid[b,d] is an exact integer sum that reveals precisely which addresses were read."""
+    B, K, F = 37, 4, 1000
+    D = 512 if dtype == torch.float32 else 64
+    _announce("addressing", mode, dtype)
+    g = torch.Generator().manual_seed(3)
+    idx = torch.randint(0, F, (B, K), generator=g)
+    if dtype == torch.float32:
+        W = (torch.arange(F).unsqueeze(1) * D + torch.arange(D)).float()  # < 2^24, exact
+    else:
+        W = ((torch.arange(F).unsqueeze(1) * 7 + torch.arange(D) * 3) % 64).float()  # exact in bf16
+    v = torch.ones(B, K)
+    args = [idx, W.to(dtype), v.to(dtype), torch.zeros(D, dtype=dtype), torch.zeros(B, D, dtype=dtype)]
+    rc, loss, resid = abi.forward(mode, *_to_dev(args))
+    assert rc == 0
+    expect = W[idx].sum(dim=1)  # exact in fp32: integer sums below 2^24
+    assert torch.equal(resid.cpu(), expect)
+
+
+@pytest.mark.parametrize("shape", [(4, 8, 16), (37, 16, 5), (64, 32, 4096), (192, 256, 512), (300, 70, 3),
+                                   (128, 64, 100000), (2048, 33, 1)])
+def test_pair_list_bit_exact(shape):
+    """begin/map equal the stable counting sort (oracle = numpy argsort(kind='stable'))."""
+    B, K, F = shape
+    _announce("csr", shape)
+    idx = torch.randint(0, F, (B, K), generator=torch.Generator().manual_seed(B + K + F))
+    rbegin, rmap = oracle.csr(idx, F)
+    for _ in range(2):  # twice: the result may not depend on how the atomics were served
+        rc, begin, mp = abi.csr_build(idx.to(DEV), F)
+        torch.cuda.synchronize()
+        assert rc == 0
+        np.testing.assert_array_equal(abi.widen_u32(begin).cpu().numpy(), rbegin.astype(np.int64))
+        np.testing.assert_array_equal(abi.widen_u32(mp).cpu().numpy(), rmap.astype(np.int64))
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_c_abi_direct(mode, dtype):
+    """Forward and backward entry points called with raw pointers; outputs start as NaN so a
+    missing zero-fill or an unwritten element shows."""
+    B, K, F, D = 48, 32, 200, 768
+    _announce("abi", mode, dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=17)
+    idx, W, v, b, t = _to_dev(args)
+    rc, loss, resid = abi.forward(mode, idx, W, v, b, t)
+    assert rc == 0
+    if mode == "hier":
+        rc, dW, dv, db = abi.hier_backward(idx, W, v, resid, 0.7)
+    else:
+        rc, dW, dv, db = abi.topk_backward(idx, W, v, resid, 0.7, dw_dtype=torch.float32)
+    assert rc == 0
+    torch.cuda.synchronize()
+    L, rW, rv, rb = oracle.loss_grads(MODES[mode], *args, grad_out=0.7)
+    tol_loss, _ = REL_TOL[dtype]
+    assert abs(loss.item() - L) <= tol_loss * abs(L)
+    # outputs here are fp32 whatever the input dtype, so the fp32 bar applies to the arithmetic
+    assert rel_err(dW.cpu(), rW) < 1e-4
+    assert rel_err(dv.cpu(), rv) < 1e-4
+    assert rel_err(db.cpu(), rb) < 1e-4
+    # resid is r_{K-1} - target
+    rW0 = W.float().cpu()[idx.cpu()] * v.float().cpu().unsqueeze(-1)
+    expect = b.float().cpu() + rW0.sum(1) - t.float().cpu()
+    assert rel_err(resid.cpu(), expect) < 1e-5
+    # untouched latents: exactly zero rows
+    untouched = np.setdiff1d(np.arange(F), idx.cpu().numpy().ravel())
+    if untouched.size:
+        assert torch.count_nonzero(dW[torch.from_numpy(untouched).to(DEV)]) == 0
+
+
+def test_hier_prezeroed_flag_and_cast():
+    args = make_inputs(16, 16, 64, 512, dtype=torch.bfloat16, seed=5)
+    idx, W, v, b, t = _to_dev(args)
+    rc, loss, resid = abi.forward("hier", idx, W, v, b, t)
+    rc1, dW1, dv1, db1 = abi.hier_backward(idx, W, v, resid, 1.0)
+    rc2, dW2, dv2, db2 = abi.hier_backward(idx, W, v, resid, 1.0, prezeroed=True)
+    assert rc == rc1 == rc2 == 0
+    assert rel_err(dW2.cpu(), dW1.cpu()) < 1e-6 and rel_err(db2.cpu(), db1.cpu()) < 1e-6
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        rc, out = abi.cast_from_f32(dW1, dt)
+        assert rc == 0
+        assert torch.equal(out, dW1.to(dt))  # same round-to-nearest-even as torch
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_loss_is_reproducible_bit_for_bit(mode):
+    args = _to_dev(make_inputs(64, 32, 224, 1024, dtype=torch.bfloat16, seed=9))
+    vals = {abi.forward(mode, *args)[1].item() for _ in range(5)}
+    assert len(vals) == 1
+
+
+def test_topk_dw_is_reproducible_bit_for_bit():
+    args = _to_dev(make_inputs(96, 32, 64, 1536, seed=9))  # F small: long groups, many collisions
+    idx, W, v, b, t = args
+    _, _, resid = abi.forward("topk", *args)
+    outs = [abi.topk_backward(idx, W, v, resid, 1.0)[1] for _ in range(3)]
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_out_of_range_index_is_flagged_not_followed(mode):
+    idx, W, v, b, t = make_inputs(8, 8, 32, 256, seed=1)
+    idx[3, 2] = 32          # == F
+    idx[5, 0] = -1
+    args = _to_dev((idx, W, v, b, t))
+    flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+    rc, loss, resid = abi.forward(mode, *args, flag=flag)
+    torch.cuda.synchronize()
+    assert rc == 0 and flag.item() == 1
+    # the offending pairs count as (latent 0, value 0): same result as zeroing them by hand
+    idx2, v2 = idx.clone(), v.clone()
+    idx2[3, 2] = idx2[5, 0] = 0
+    v2[3, 2] = v2[5, 0] = 0
+    L, *_ = oracle.loss_grads(MODES[mode], idx2, W, v2, b, t, want_grads=False)
+    assert abs(loss.item() - L) <= 1e-5 * abs(L)
+    # python layer: the check raises IndexError and clears the flag
+    try:
+        flex.check_index_flag()
+    except IndexError:
+        pass
+    FUSED[mode](*args)
+    with pytest.raises(IndexError):
+        flex.check_index_flag()
+    flex.check_index_flag()
+
+
+def test_topk_target_gradient():
+    args = make_inputs(16, 8, 40, 256, seed=2)
+    idx, W, v, b, t = _to_dev(args)
+    t.requires_grad_()
+    W.requires_grad_()
+    flex.triton_topk_sae_loss(idx, W, v, b, t).backward()
+    tr = args[4].double().requires_grad_()
+    oracle.torch_loss(oracle.TOPK, args[0], args[1].double(), args[2].double(), args[3].double(), tr,
+                      compute_dtype=torch.float64).backward()
+    assert rel_err(t.grad.cpu(), tr.grad) < 1e-4
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_non_contiguous_inputs(mode):
+    idx, W, v, b, t = make_inputs(16, 8, 40, 256, seed=4)
+    Wd = torch.empty(40, 512, device=DEV)[:, ::2]
+    Wd.copy_(W)
+    td = torch.empty(256, 16, device=DEV).t()
+    td.copy_(t)
+    assert not Wd.is_contiguous() and not td.is_contiguous()
+    loss = FUSED[mode](idx.to(DEV), Wd, v.to(DEV), b.to(DEV), td)
+    L, *_ = oracle.loss_grads(MODES[mode], idx, W, v, b, t, want_grads=False)
+    assert abs(loss.item() - L) <= 1e-5 * abs(L)
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_opcheck_and_compile(mode):
+    args = _to_dev(make_inputs(16, 8, 40, 256, seed=6))
+    idx, W, v, b, t = args
+    W.requires_grad_()
+    v.requires_grad_()
+    b.requires_grad_()
+    op = torch.ops.flexsae_amd.hier_fwd if mode == "hier" else torch.ops.flexsae_amd.topk_fwd
+    torch.library.opcheck(op, (idx, W, v, b, t),
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+    eager = FUSED[mode](idx, W, v, b, t)
+    compiled = torch.compile(lambda *a: FUSED[mode](*a) * 2.0, fullgraph=True, backend="aot_eager")(idx, W, v, b, t)
+    assert abs(compiled.item() - 2.0 * eager.item()) <= 1e-6 * abs(eager.item())
+    compiled.backward()
+    assert W.grad is not None and v.grad is not None and b.grad is not None
