@@ -52,7 +52,10 @@ def _check_against_oracle(mode, args_cpu, dtype, grad_out, got, ref_tols=True):
     assert dW.dtype == dtype and dv.dtype == dtype and db.dtype == dtype
     for name, g, r in (("dW", dW, rW), ("dvals", dv, rv), ("dbias", db, rb)):
         err = rel_err(g.float().cpu(), r)
-        assert err <= tol_grad, f"{name}: rel err {err:.3e} > {tol_grad}"
+        # what rounding the exact gradient to the leaf dtype costs by itself (fp16 gradients of
+        # magnitude 2/(B*K*D) are subnormal, so this can exceed the arithmetic tolerance)
+        quant = rel_err(torch.from_numpy(r).to(dtype).double(), r)
+        assert err <= tol_grad + 1.5 * quant, f"{name}: rel err {err:.3e} > {tol_grad} + 1.5*{quant:.3e}"
     if ref_tols:
         tols = DTYPE_TO_TOLS[dtype]
         torch.testing.assert_close(loss.cpu(), torch.tensor(L, dtype=torch.float32), **tols)
