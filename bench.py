@@ -38,6 +38,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_k128", choices=sorted(WORKLOADS))
+    ap.add_argument("--shape", default="", help="override B,K,F,D of the workload (tuning aid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU-baseline sample (0 = auto)")
     return ap.parse_args()
@@ -187,6 +188,8 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     B, K, F, D, dt_name, dist, w_std = WORKLOADS[args.workload]
+    if args.shape:
+        B, K, F, D = (int(x) for x in args.shape.split(","))
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[dt_name]
     es = 2 if dtype == torch.bfloat16 else 4
     inputs = make_inputs(torch, B, K, F, D, dtype, dist, w_std, dev)
@@ -222,31 +225,30 @@ def main():
     loss = torch.empty(1, dtype=torch.float32, device=dev)
     resid = torch.empty(B, D, dtype=torch.float32, device=dev)
     g1 = torch.ones(1, dtype=torch.float32, device=dev)
-    dW_acc = torch.empty(F, D, dtype=torch.float32, device=dev)
     dvals = torch.empty(B, K, dtype=torch.float32, device=dev)
     dbias = torch.empty(D, dtype=torch.float32, device=dev)
+    dW = torch.empty(F, D, dtype=dtype, device=dev)
+    scratch = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
+    slice_cols = max(1, scratch // (B * K * (2 if dtype == torch.bfloat16 else 4)))
+    bws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+    bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
 
     def fwd_launch():
         _lib.check(lib.flexsae_hier_fwd(ctypes.byref(sh), p(idx), p(W), p(v), p(b), p(t), p(loss), p(resid), p(ws),
                                         ws_bytes, None, st()), "flexsae_hier_fwd")
 
-    def bwd_prepare():
-        dW_acc.zero_()
-        dvals.zero_()
-        dbias.zero_()
-
     def bwd_launch():
-        _lib.check(lib.flexsae_hier_bwd(ctypes.byref(sh), p(idx), p(W), p(v), p(resid), p(g1), p(dW_acc), p(dvals),
-                                        p(dbias), _lib.BWD_OUTPUTS_PREZEROED, None, st()), "flexsae_hier_bwd")
+        _lib.check(lib.flexsae_hier_bwd(ctypes.byref(sh), p(idx), p(W), p(v), p(resid), p(g1), p(dW), DT[dtype],
+                                        p(dvals), p(dbias), p(bws), bws_bytes, 0, None, st()), "flexsae_hier_bwd")
 
     fwd_k_ms = time_kernel_events(torch, lambda: None, fwd_launch, args.steps, args.warmup)
-    bwd_k_ms = time_kernel_events(torch, bwd_prepare, bwd_launch, args.steps, args.warmup)
-    del dW_acc
+    bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
+    del dW, bws
 
     def gbps(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
-    dominant = "hier_bwd_kernel" if bwd_k_ms >= fwd_k_ms else "sae_fwd_kernel(hier)"
+    dominant = "flexsae_hier_bwd (pair list + sweep + segment reduce)" if bwd_k_ms >= fwd_k_ms else "sae_fwd_kernel(hier)"
     dom_bytes = abytes["hier_bwd_kernel"] if bwd_k_ms >= fwd_k_ms else abytes["fwd_kernel"]
     dom_ms = max(bwd_k_ms, fwd_k_ms)
     roofline = {
@@ -283,7 +285,7 @@ def main():
         "kernels": {
             "sae_fwd_kernel(hier)": {"ms": round(fwd_k_ms, 4), "algorithmic_bytes": abytes["fwd_kernel"],
                                      "GBps": round(gbps(abytes["fwd_kernel"], fwd_k_ms), 1)},
-            "hier_bwd_kernel": {"ms": round(bwd_k_ms, 4), "algorithmic_bytes": abytes["hier_bwd_kernel"],
+            "flexsae_hier_bwd": {"ms": round(bwd_k_ms, 4), "algorithmic_bytes": abytes["hier_bwd_kernel"],
                                 "GBps": round(gbps(abytes["hier_bwd_kernel"], bwd_k_ms), 1)},
         },
         "topk": {"ms_per_step": round(topk_ms, 4), "algorithmic_bytes": abytes["topk_step"],

@@ -24,12 +24,23 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
   return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
 
-// round-to-nearest-even, NaN kept quiet
+// round-to-nearest-even through the hardware converter (v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  const __bf16 h = static_cast<__bf16>(f);
+  uint16_t u;
+  __builtin_memcpy(&u, &h, 2);
+  return u;
+}
+
+// two floats -> two bf16 packed in one dword (element 0 in the low half), one instruction
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 x = {lo, hi};
+  const bf16x2 y = __builtin_convertvector(x, bf16x2);
+  uint32_t u;
+  __builtin_memcpy(&u, &y, 4);
+  return u;
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
@@ -90,7 +101,14 @@ template <typename T, int VEC>
 __device__ __forceinline__ void store_vec(void *base, int64_t off, const float (&x)[VEC]) {
   using S = typename Traits<T>::store_t;
   S *p = static_cast<S *>(base) + off;
-  if constexpr (VEC == 1) {
+  if constexpr (Traits<T>::dtype == FLEXSAE_BF16 && VEC == 2) {
+    *reinterpret_cast<uint32_t *>(p) = f32x2_to_bf16x2_bits(x[0], x[1]);
+  } else if constexpr (Traits<T>::dtype == FLEXSAE_BF16 && VEC > 2) {
+    vec_t<uint32_t, VEC / 2> v;
+#pragma unroll
+    for (int i = 0; i < VEC / 2; ++i) v[i] = f32x2_to_bf16x2_bits(x[2 * i], x[2 * i + 1]);
+    *reinterpret_cast<vec_t<uint32_t, VEC / 2> *>(p) = v;
+  } else if constexpr (VEC == 1) {
     *p = Traits<T>::down(x[0]);
   } else {
     vec_t<S, VEC> v;

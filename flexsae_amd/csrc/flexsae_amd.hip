@@ -5,6 +5,7 @@
 #include "common.hpp"
 #include "fwd_kernels.hpp"
 #include "hier_bwd_kernels.hpp"
+#include "segment_kernels.hpp"
 #include "topk_bwd_kernels.hpp"
 
 using namespace flexsae;
@@ -61,7 +62,7 @@ struct FwdPlan {
 FwdPlan plan_fwd(const flexsae_shape *s, const void *weight, const void *target, const void *bias,
                  const float *resid) {
   const size_t es = dtype_size(s->weight_dtype);
-  int vec = pick_vec(s->D, es, weight, es == 4 ? 4 : 8);
+  int vec = pick_vec(s->D, es, weight, 4);  // 256-column tiles measured faster than 512
   // resid is stored with fp32 vectors of the same width, target/bias are read with the
   // weight's vector type when they share its dtype
   if (s->target_dtype == s->weight_dtype && !aligned(target, vec * es)) vec = 1;
@@ -224,6 +225,192 @@ void launch_topk_bwd_g(const flexsae_shape *s, const uint32_t *begin, const uint
   }
 }
 
+// Scratch of the pair-list construction, carved out of one workspace:
+// cursor[F] | scan block sums[ceil(F/kScanBlockElems)] | long_count (one aligned slot) |
+// long_list[B*K/65 + 1]
+struct CsrScratch {
+  uint32_t *cursor;
+  uint32_t *block_sums;
+  uint32_t *long_count;
+  uint32_t *long_list;
+};
+
+size_t csr_scan_sums_bytes(int64_t F) {
+  return round_up(static_cast<size_t>(ceil_div(F, kScanBlockElems)) * 4, kAlign);
+}
+
+CsrScratch carve_csr_scratch(void *workspace, int64_t F) {
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
+  CsrScratch sc;
+  sc.cursor = reinterpret_cast<uint32_t *>(ws);
+  ws += round_up(static_cast<size_t>(F) * 4, kAlign);
+  sc.block_sums = reinterpret_cast<uint32_t *>(ws);
+  ws += csr_scan_sums_bytes(F);
+  sc.long_count = reinterpret_cast<uint32_t *>(ws);
+  sc.long_list = reinterpret_cast<uint32_t *>(ws + kAlign);
+  return sc;
+}
+
+void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, uint32_t *begin,
+                      uint32_t *map, const CsrScratch &sc, int *status_flag, hipStream_t st) {
+  const int64_t n_pairs = B * K;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(F + 1, 256, 4096)), dim3(256), 0, st, begin,
+                     F + 1, 0u);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, sc.long_count,
+                     static_cast<int64_t>(1), 0u);
+  hipLaunchKernelGGL(csr_count_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st,
+                     indices, n_pairs, F, begin, status_flag);
+  const unsigned scan_blocks = static_cast<unsigned>(ceil_div(F, kScanBlockElems));
+  hipLaunchKernelGGL(csr_scan_sums_kernel, dim3(scan_blocks), dim3(kScanThreads), 0, st, begin, F,
+                     sc.block_sums);
+  hipLaunchKernelGGL(csr_scan_apply_kernel, dim3(scan_blocks), dim3(kScanThreads), 0, st, begin,
+                     sc.cursor, F, sc.block_sums);
+  hipLaunchKernelGGL(csr_fill_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, indices,
+                     n_pairs, F, sc.cursor, map);
+  hipLaunchKernelGGL(csr_sort_short_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(F, kWavesPerBlock))), dim3(kBlock), 0, st,
+                     begin, map, F, sc.long_count, sc.long_list);
+  hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(256), 0, st, begin, map, sc.long_count,
+                     sc.long_list);
+}
+
+// ---- two-phase hierarchical backward: workspace plan -----------------------------------
+
+struct HierBwdPlan {
+  int vec;                 // columns per lane
+  int tile;                // 64 * vec columns per wavefront
+  size_t p_size;           // bytes per element of the contribution matrix P
+  int64_t d_pad;           // D rounded up to a whole number of tiles
+  size_t n_pairs;          // B * K
+  size_t n_rows;           // B
+  size_t n_partial_rows;   // upper bound on the number of 64-pair chunks of long latents
+  size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_sfinal, off_colsum, off_partial;  // per-slice buffers follow
+  size_t fixed_bytes;      // everything that does not depend on the slice width
+};
+
+HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
+  HierBwdPlan p;
+  p.vec = (s->D % 4 == 0) ? 4 : (s->D % 2 == 0) ? 2 : 1;
+  p.tile = kWave * p.vec;
+  p.p_size = (s->weight_dtype == FLEXSAE_BF16) ? 2 : 4;  // bf16 weights: bf16 contributions
+  p.d_pad = ceil_div(s->D, p.tile) * p.tile;
+  p.n_pairs = static_cast<size_t>(s->B) * static_cast<size_t>(s->K);
+  p.n_rows = static_cast<size_t>(s->B);
+  p.n_partial_rows = p.n_pairs / kSegChunk + p.n_pairs / 65 + 2;
+  size_t off = 0;
+  p.off_begin = off;
+  off += round_up(static_cast<size_t>(s->F + 1) * 4, kAlign);
+  p.off_map = off;
+  off += round_up(p.n_pairs * 4, kAlign);
+  p.off_slot = off;
+  off += round_up(p.n_pairs * 4, kAlign);
+  p.off_csr = off;
+  off += flexsae_csr_workspace_bytes(s->B, s->K, s->F);
+  p.off_chunk = off;
+  off += round_up((p.n_pairs / 65 + 2) * 4, kAlign);
+  p.off_sfinal = off;  // S_{b,0} of every row, [B, d_pad] fp32: dbias is its column sum
+  off += round_up(p.n_rows * static_cast<size_t>(p.d_pad) * 4, kAlign);
+  p.off_colsum = off;  // partial column sums, [ceil(B/64), D] fp32
+  off += round_up(static_cast<size_t>(ceil_div(s->B, kColsumRows)) * static_cast<size_t>(s->D) * 4, kAlign);
+  p.off_partial = off;
+  p.fixed_bytes = off;
+  return p;
+}
+
+// per-slice buffers after the fixed part: chunk partials[n_partial_rows, w] | P[B*K, w]
+size_t hier_partial_bytes(const HierBwdPlan &p, int64_t slice_w) {
+  return round_up(p.n_partial_rows * static_cast<size_t>(slice_w) * 4, kAlign);
+}
+
+size_t hier_bwd_bytes(const HierBwdPlan &p, int64_t slice_w) {
+  return p.fixed_bytes + hier_partial_bytes(p, slice_w) +
+         round_up(p.n_pairs * static_cast<size_t>(slice_w) * p.p_size, kAlign);
+}
+
+template <typename WT, typename PT, typename GT, int VEC>
+void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t slice_w,
+                        const int64_t *indices, const void *weight, const void *vals,
+                        const float *resid, const float *grad_out, float coef, void *dW,
+                        float *dvals, float *dbias, uint8_t *ws, int *status_flag, hipStream_t st) {
+  const uint32_t *begin = reinterpret_cast<const uint32_t *>(ws + pl.off_begin);
+  const uint32_t *slot = reinterpret_cast<const uint32_t *>(ws + pl.off_slot);
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
+  uint32_t *chunk_begin = reinterpret_cast<uint32_t *>(ws + pl.off_chunk);
+  float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
+  void *P = ws + pl.off_partial + hier_partial_bytes(pl, slice_w);
+  float *s_final = reinterpret_cast<float *>(ws + pl.off_sfinal);
+  float *colsum_part = reinterpret_cast<float *>(ws + pl.off_colsum);
+  const int n_chunks = static_cast<int>(ceil_div(s->B, kColsumRows));
+  const int d_pad = static_cast<int>(pl.d_pad);
+  const int K = static_cast<int>(s->K), D = static_cast<int>(s->D);
+  const int sw = static_cast<int>(slice_w);
+  for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
+    const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
+    const int tps = static_cast<int>(cols / pl.tile);
+    const int64_t sweep_items = s->B * tps;
+    hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, 8>),
+                       dim3(static_cast<unsigned>(ceil_div(sweep_items, kWavesPerBlock))), dim3(kBlock),
+                       0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dvals,
+                       s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F, D);
+    hipLaunchKernelGGL((seg_reduce_short_kernel<PT, GT, VEC, 8>),
+                       dim3(static_cast<unsigned>(ceil_div(s->F, kWavesPerBlock))), dim3(kBlock), 0, st,
+                       begin, P, dW, s->F, tps, static_cast<int>(col0), sw, D);
+    hipLaunchKernelGGL((seg_reduce_long_kernel<PT, VEC, 8>), dim3(1024), dim3(kBlock), 0, st, begin,
+                       sc.long_count, sc.long_list, chunk_begin, P, partial, tps, sw);
+    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
+                       sc.long_count, sc.long_list, chunk_begin, partial, dW, tps,
+                       static_cast<int>(col0), sw, D);
+  }
+  // dbias = column sums of s_final over the rows, in a fixed order
+  hipLaunchKernelGGL(colsum_partial_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
+                     0, st, s_final, s->B, static_cast<int64_t>(d_pad), D, colsum_part);
+  hipLaunchKernelGGL(colsum_final_kernel, dim3(static_cast<unsigned>(ceil_div(D, 256))), dim3(256), 0, st,
+                     colsum_part, n_chunks, D, static_cast<const float *>(nullptr), 1.0f, dbias);
+}
+
+template <typename WT, typename PT, int VEC>
+void launch_hier_slices_g(const flexsae_shape *s, const HierBwdPlan &pl, int64_t slice_w,
+                          const int64_t *indices, const void *weight, const void *vals,
+                          const float *resid, const float *grad_out, float coef, void *dW,
+                          int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int *status_flag,
+                          hipStream_t st) {
+  switch (dW_dtype) {
+    case FLEXSAE_F32:
+      launch_hier_slices<WT, PT, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
+                                             coef, dW, dvals, dbias, ws, status_flag, st);
+      break;
+    case FLEXSAE_BF16:
+      launch_hier_slices<WT, PT, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
+                                              coef, dW, dvals, dbias, ws, status_flag, st);
+      break;
+    default:
+      launch_hier_slices<WT, PT, f16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
+                                             coef, dW, dvals, dbias, ws, status_flag, st);
+  }
+}
+
+template <int VEC>
+void launch_hier_slices_w(const flexsae_shape *s, const HierBwdPlan &pl, int64_t slice_w,
+                          const int64_t *indices, const void *weight, const void *vals,
+                          const float *resid, const float *grad_out, float coef, void *dW,
+                          int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int *status_flag,
+                          hipStream_t st) {
+  switch (s->weight_dtype) {
+    case FLEXSAE_F32:
+      launch_hier_slices_g<float, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
+                                              coef, dW, dW_dtype, dvals, dbias, ws, status_flag, st);
+      break;
+    case FLEXSAE_BF16:
+      launch_hier_slices_g<bf16_t, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
+                                                coef, dW, dW_dtype, dvals, dbias, ws, status_flag, st);
+      break;
+    default:
+      launch_hier_slices_g<f16_t, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
+                                              coef, dW, dW_dtype, dvals, dbias, ws, status_flag, st);
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -271,9 +458,10 @@ int flexsae_topk_fwd(const flexsae_shape *shape, const int64_t *indices, const v
                         workspace_bytes, status_flag, stream);
 }
 
-int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void *weight,
-                     const void *vals, const float *resid, const float *grad_out, float *dW_acc,
-                     float *dvals, float *dbias, int flags, int *status_flag, void *stream) {
+int flexsae_hier_bwd_atomic(const flexsae_shape *s, const int64_t *indices, const void *weight,
+                            const void *vals, const float *resid, const float *grad_out,
+                            float *dW_acc, float *dvals, float *dbias, int flags, int *status_flag,
+                            void *stream) {
   int rc = check_shape(s);
   if (rc != FLEXSAE_OK) return rc;
   if (!indices || !weight || !vals || !resid || !grad_out || !dW_acc || !dvals || !dbias)
@@ -306,10 +494,65 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   return launch_status();
 }
 
+size_t flexsae_hier_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_cols) {
+  if (check_shape(s) != FLEXSAE_OK) return 0;
+  const HierBwdPlan pl = plan_hier_bwd(s);
+  int64_t sw = slice_cols <= 0 ? pl.tile : ceil_div(slice_cols, pl.tile) * pl.tile;
+  if (sw > pl.d_pad) sw = pl.d_pad;
+  return hier_bwd_bytes(pl, sw);
+}
+
+int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void *weight,
+                     const void *vals, const float *resid, const float *grad_out, void *dW,
+                     int dW_dtype, float *dvals, float *dbias, void *workspace,
+                     size_t workspace_bytes, int flags, int *status_flag, void *stream) {
+  int rc = check_shape(s);
+  if (rc != FLEXSAE_OK) return rc;
+  if (!indices || !weight || !vals || !resid || !grad_out || !dW || !dvals || !dbias ||
+      !valid_dtype(dW_dtype))
+    return FLEXSAE_ERR_INVALID_ARGUMENT;
+  const HierBwdPlan pl = plan_hier_bwd(s);
+  if (!aligned(indices, 8) || !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
+      !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.vec * 4) ||
+      !aligned(grad_out, 4) || !aligned(dW, pl.vec * dtype_size(dW_dtype)) || !aligned(dvals, 16) ||
+      !aligned(dbias, 16))
+    return FLEXSAE_ERR_ALIGNMENT;
+  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, pl.tile))
+    return FLEXSAE_ERR_WORKSPACE;
+  // widest slice (whole tiles) the workspace can hold
+  int64_t slice_w = pl.tile;
+  while (slice_w + pl.tile <= pl.d_pad && hier_bwd_bytes(pl, slice_w + pl.tile) <= workspace_bytes)
+    slice_w += pl.tile;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
+  if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) zero_f32(dvals, s->B * s->K, st);
+  uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
+  uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
+  csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
+  hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
+                     s->B * s->K, reinterpret_cast<uint32_t *>(ws + pl.off_slot));
+  hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
+                     sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+  const float coef = static_cast<float>(
+      2.0 / (static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D)));
+  if (pl.vec == 4) {
+    launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, resid, grad_out, coef, dW, dW_dtype,
+                            dvals, dbias, ws, status_flag, st);
+  } else if (pl.vec == 2) {
+    launch_hier_slices_w<2>(s, pl, slice_w, indices, weight, vals, resid, grad_out, coef, dW, dW_dtype,
+                            dvals, dbias, ws, status_flag, st);
+  } else {
+    launch_hier_slices_w<1>(s, pl, slice_w, indices, weight, vals, resid, grad_out, coef, dW, dW_dtype,
+                            dvals, dbias, ws, status_flag, st);
+  }
+  return launch_status();
+}
+
 size_t flexsae_csr_workspace_bytes(int64_t B, int64_t K, int64_t F) {
   if (B <= 0 || K <= 0 || F <= 0) return 0;
-  // cursor[F] | long_count (padded) | long_list[B*K/65 + 1]
-  return round_up(static_cast<size_t>(F) * 4, kAlign) + kAlign +
+  // cursor[F] | scan block sums | long_count (padded) | long_list[B*K/65 + 1]
+  return round_up(static_cast<size_t>(F) * 4, kAlign) + csr_scan_sums_bytes(F) + kAlign +
          round_up((static_cast<size_t>(B) * static_cast<size_t>(K) / 65 + 1) * 4, kAlign);
 }
 
@@ -322,32 +565,20 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
   if (!workspace || workspace_bytes < flexsae_csr_workspace_bytes(B, K, F) ||
       !aligned(workspace, kAlign))
     return FLEXSAE_ERR_WORKSPACE;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  const int64_t n_pairs = B * K;
-  uint8_t *ws = static_cast<uint8_t *>(workspace);
-  uint32_t *cursor = reinterpret_cast<uint32_t *>(ws);
-  uint32_t *long_count = reinterpret_cast<uint32_t *>(ws + round_up(static_cast<size_t>(F) * 4, kAlign));
-  uint32_t *long_list = reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(long_count) + kAlign);
-
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(F + 1, 256, 4096)), dim3(256), 0, st, begin,
-                     F + 1, 0u);
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, long_count, static_cast<int64_t>(1), 0u);
-  hipLaunchKernelGGL(csr_count_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st,
-                     indices, n_pairs, F, begin, status_flag);
-  hipLaunchKernelGGL(csr_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, begin, cursor, F);
-  hipLaunchKernelGGL(csr_fill_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, indices,
-                     n_pairs, F, cursor, map);
-  hipLaunchKernelGGL(csr_sort_short_kernel, dim3(static_cast<unsigned>(ceil_div(F, kWavesPerBlock))),
-                     dim3(kBlock), 0, st, begin, map, F, long_count, long_list);
-  hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(256), 0, st, begin, map, long_count,
-                     long_list);
+  const CsrScratch sc = carve_csr_scratch(workspace, F);
+  csr_build_launch(indices, B, K, F, begin, map, sc, status_flag, static_cast<hipStream_t>(stream));
   return launch_status();
+}
+
+size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *s) {
+  if (check_shape(s) != FLEXSAE_OK) return 0;
+  return round_up(static_cast<size_t>(ceil_div(s->B, kColsumRows)) * static_cast<size_t>(s->D) * 4, kAlign);
 }
 
 int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32_t *map,
                      const void *weight, const void *vals, const float *resid,
                      const float *grad_out, void *dW, int dW_dtype, float *dvals, float *dbias,
-                     int flags, void *stream) {
+                     void *workspace, size_t workspace_bytes, int flags, void *stream) {
   int rc = check_shape(s);
   if (rc != FLEXSAE_OK) return rc;
   if (!begin || !map || !weight || !vals || !resid || !grad_out || !dW || !dvals || !dbias ||
@@ -355,13 +586,12 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
     return FLEXSAE_ERR_INVALID_ARGUMENT;
   if (!aligned(begin, 4) || !aligned(map, 4) || !aligned(weight, dtype_size(s->weight_dtype)) ||
       !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, 4) || !aligned(grad_out, 4) ||
-      !aligned(dW, dtype_size(dW_dtype)) || !aligned(dvals, 16) || !aligned(dbias, 16))
+      !aligned(dW, dtype_size(dW_dtype)) || !aligned(dvals, 16) || !aligned(dbias, 4))
     return FLEXSAE_ERR_ALIGNMENT;
+  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < flexsae_topk_bwd_workspace_bytes(s))
+    return FLEXSAE_ERR_WORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) {
-    zero_f32(dvals, s->B * s->K, st);
-    zero_f32(dbias, s->D, st);
-  }
+  if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) zero_f32(dvals, s->B * s->K, st);
   const float coef =
       static_cast<float>(2.0 / (static_cast<double>(s->B) * static_cast<double>(s->D)));
   // vector width: resid rows are read as fp32 vectors, weight/dW rows in their own types
@@ -386,12 +616,15 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
   }
   rc = launch_status();
   if (rc != FLEXSAE_OK) return rc;
-  const int rows_per_block = 64;
-  hipLaunchKernelGGL(colsum_kernel,
-                     dim3(static_cast<unsigned>(ceil_div(s->D, 256)),
-                          static_cast<unsigned>(ceil_div(s->B, rows_per_block))),
-                     dim3(256), 0, st, resid, grad_out, coef, dbias, s->B, static_cast<int>(s->D),
-                     rows_per_block);
+  // dbias = coef * grad_out * column sums of resid, in a fixed order
+  float *colsum_part = static_cast<float *>(workspace);
+  const int n_chunks = static_cast<int>(ceil_div(s->B, kColsumRows));
+  const int D = static_cast<int>(s->D);
+  hipLaunchKernelGGL(colsum_partial_kernel,
+                     dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
+                     0, st, resid, s->B, s->D, D, colsum_part);
+  hipLaunchKernelGGL(colsum_final_kernel, dim3(static_cast<unsigned>(ceil_div(D, 256))), dim3(256), 0, st,
+                     colsum_part, n_chunks, D, grad_out, coef, dbias);
   return launch_status();
 }
 

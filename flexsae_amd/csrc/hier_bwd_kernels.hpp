@@ -106,3 +106,110 @@ __global__ __launch_bounds__(256) void hier_bwd_kernel(
 }
 
 }  // namespace flexsae
+
+namespace flexsae {
+
+// Sweep kernel of the two-phase backward.  Same reverse walk as hier_bwd_kernel, but the
+// per-pair contribution vals_k * S is STORED instead of being added to dW with atomics (the
+// L2 atomic units retire about one fp32 per clock and channel, far below what the walk can
+// produce).  The contribution of pair p goes to row slot[p] of P, slot[] being the pair's
+// position in the latent-major pair list, so that all rows of one latent are adjacent and a
+// segment reduction (segment_kernels.hpp) can stream them.  Only the columns
+// [col0, col0 + tps*64*VEC) of the problem (one "slice") are handled per launch, so P needs
+// B*K*slice_width elements.  dvals partial dot products are added across tiles with atomics
+// (one address per pair and tile: no contention).
+//
+// One wavefront per (tile of the slice, row b), tile-major: the wavefronts in flight at any
+// moment gather from the same 64*VEC-column slice of W, which is small enough to stay in the
+// on-chip caches while it is being reused by every row.  Lane l owns VEC consecutive columns,
+// so the gathered weight piece and the stored contribution are one vector access per lane.
+template <typename WT, typename PT, int VEC, int U>
+__global__ __launch_bounds__(256) void hier_sweep_kernel(
+    const int64_t *__restrict__ indices, const void *__restrict__ weight,
+    const void *__restrict__ vals, int vals_dtype, const float *__restrict__ resid,
+    const float *__restrict__ grad_out, float coef, const uint32_t *__restrict__ slot,
+    void *__restrict__ P, float *__restrict__ dvals, float *__restrict__ s_final, int s_final_ld,
+    int *status_flag, int64_t n_items, int64_t B, int col0, int slice_w, int K, int64_t F,
+    int D) {
+  const int lane = lane_id();
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+  if (item >= n_items) return;  // uniform per wavefront
+  const int t = static_cast<int>(item / B);
+  const int64_t b = item - static_cast<int64_t>(t) * B;
+  const int pc = t * (kWave * VEC) + lane * VEC;  // column inside the slice
+  const int d0 = col0 + pc;
+  const bool active = d0 < D;
+  const int dsafe = active ? d0 : 0;
+  const float scale = coef * grad_out[0];
+
+  float e[VEC], S[VEC];
+  load_vec<float, VEC>(resid, b * D + dsafe, e);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) S[i] = 0.f;
+
+  const int64_t pair0 = b * K;
+  for (int k0 = ((K - 1) / kWave) * kWave; k0 >= 0; k0 -= kWave) {
+    const int kk = k0 + lane;
+    int64_t my_idx = 0;
+    float my_val = 0.f;
+    int my_slot = 0;
+    if (kk < K) {
+      my_idx = indices[pair0 + kk];
+      my_val = load_scalar(vals, vals_dtype, pair0 + kk);
+      my_slot = static_cast<int>(slot[pair0 + kk]);
+    }
+    if (static_cast<uint64_t>(my_idx) >= static_cast<uint64_t>(F)) {
+      if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
+      my_idx = 0;
+      my_val = 0.f;
+    }
+    const int my_row = static_cast<int>(my_idx);
+    const int n = (K - k0) < kWave ? (K - k0) : kWave;  // uniform
+    float my_dval = 0.f;
+
+    auto step = [&](int j, const float(&w)[VEC]) {
+      const float v = bcast_f32(my_val, j);
+      const int64_t prow = static_cast<uint32_t>(bcast_i32(my_slot, j));
+      float contrib[VEC];
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        S[i] = fmaf(scale, e[i], S[i]);
+        contrib[i] = S[i] * v;
+        dot = fmaf(w[i], S[i], dot);
+        e[i] = fmaf(-w[i], v, e[i]);
+      }
+      if (active) store_vec<PT, VEC>(P, prow * slice_w + pc, contrib);
+      dot = wave_sum_bcast(active ? dot : 0.f);
+      if (lane == j) my_dval = dot;
+    };
+
+    int j = n - 1;
+    for (; j - (U - 1) >= 0; j -= U) {
+      float w[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t row = bcast_i32(my_row, j - u);
+        load_vec<WT, VEC>(weight, row * D + dsafe, w[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) step(j - u, w[u]);
+    }
+    for (; j >= 0; --j) {
+      float w[VEC];
+      const int64_t row = bcast_i32(my_row, j);
+      load_vec<WT, VEC>(weight, row * D + dsafe, w);
+      step(j, w);
+    }
+    if (kk < K) unsafeAtomicAdd(dvals + pair0 + kk, my_dval);
+  }
+  // the row's total S_{b,0} (its share of dbias) goes to s_final[b, column]; a column sum over
+  // b follows (thousands of atomics per dbias element would serialise instead)
+  if (!active) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) S[i] = 0.f;
+  }
+  store_vec<float, VEC>(s_final, b * s_final_ld + col0 + pc, S);
+}
+
+}  // namespace flexsae

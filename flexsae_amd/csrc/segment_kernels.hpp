@@ -1,0 +1,158 @@
+// Latent-major segment reduction: out[f, slice] = sum of the rows [begin[f], begin[f+1]) of
+// P[., slice] (rows of one latent are adjacent), with fp32 accumulation and one write per
+// output element.  Short groups (<= 64 rows) are reduced by one wavefront; long ones are cut
+// into chunks of 64 rows whose fp32 partial sums are combined by a second kernel, so a hot
+// latent is spread over many wavefronts and the summation order stays fixed (deterministic).
+#pragma once
+
+#include "common.hpp"
+
+namespace flexsae {
+
+constexpr int kSegChunk = 64;  // rows per chunk; groups longer than this count as "long"
+
+// acc += sum of rows [r0, r0+n) of X (row stride `ld` elements) over the lane's VEC columns at pc
+template <typename PT, int VEC, int U>
+__device__ __forceinline__ void accumulate_rows(const void *__restrict__ X, int64_t r0, int n,
+                                                int64_t ld, int pc, float (&acc)[VEC]) {
+  int j = 0;
+  for (; j + U <= n; j += U) {
+    float x[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) load_vec<PT, VEC>(X, (r0 + j + u) * ld + pc, x[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[i] += x[u][i];
+  }
+  for (; j < n; ++j) {
+    float x[VEC];
+    load_vec<PT, VEC>(X, (r0 + j) * ld + pc, x);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] += x[i];
+  }
+}
+
+// One wavefront per latent; it walks the tiles of the slice (64*VEC columns each).  Latents
+// with more than kSegChunk rows are left to the long path; latents without rows get zeros.
+template <typename PT, typename GT, int VEC, int U>
+__global__ __launch_bounds__(256) void seg_reduce_short_kernel(
+    const uint32_t *__restrict__ begin, const void *__restrict__ P, void *__restrict__ out,
+    int64_t F, int tps, int col0, int slice_w, int D) {
+  const int lane = lane_id();
+  const int64_t f = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+  if (f >= F) return;  // uniform per wavefront
+  const uint32_t s0 = begin[f];
+  const uint32_t n = begin[f + 1] - s0;
+  if (n > static_cast<uint32_t>(kSegChunk)) return;
+  for (int t = 0; t < tps; ++t) {
+    const int pc = t * (kWave * VEC) + lane * VEC;
+    const int d0 = col0 + pc;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    accumulate_rows<PT, VEC, U>(P, s0, static_cast<int>(n), slice_w, pc, acc);
+    if (d0 < D) store_vec<GT, VEC>(out, f * D + d0, acc);
+  }
+}
+
+// chunk_begin[i] = number of chunks of the long latents before long_list[i]
+// (chunk_begin[n_long] = total); single block.
+__global__ __launch_bounds__(1024) void seg_chunk_table_kernel(const uint32_t *__restrict__ begin,
+                                                               const uint32_t *__restrict__ long_count,
+                                                               const uint32_t *__restrict__ long_list,
+                                                               uint32_t *__restrict__ chunk_begin) {
+  __shared__ uint32_t wave_tot[1024 / kWave];
+  __shared__ uint32_t carry_s;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid >> 6;
+  const uint32_t n_long = *long_count;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (uint32_t base = 0; base < n_long; base += 1024) {
+    const uint32_t i = base + tid;
+    uint32_t c = 0;
+    if (i < n_long) {
+      const uint32_t f = long_list[i];
+      c = (begin[f + 1] - begin[f] + kSegChunk - 1) / kSegChunk;
+    }
+    uint32_t inc = c;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const uint32_t y = __shfl_up(inc, off, kWave);
+      if (lane >= off) inc += y;
+    }
+    if (lane == kWave - 1) wave_tot[wv] = inc;
+    __syncthreads();
+    uint32_t wave_off = 0;
+    for (int w = 0; w < wv; ++w) wave_off += wave_tot[w];
+    const uint32_t excl = carry_s + wave_off + inc - c;
+    if (i < n_long) chunk_begin[i] = excl;
+    __syncthreads();
+    if (tid == 1023) carry_s = excl + c;
+    __syncthreads();
+  }
+  if (tid == 0) chunk_begin[n_long] = carry_s;
+}
+
+// Long latents, step 1: every (chunk, tile) is reduced by one wavefront into
+// partial[chunk, slice] (fp32).  Fixed-size grid; wavefronts stride over the work list, whose
+// length is only known on the device.
+template <typename PT, int VEC, int U>
+__global__ __launch_bounds__(256) void seg_reduce_long_kernel(
+    const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
+    const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
+    const void *__restrict__ P, float *__restrict__ partial, int tps, int slice_w) {
+  const int lane = lane_id();
+  const uint32_t n_long = *long_count;
+  if (n_long == 0) return;
+  const int64_t total = static_cast<int64_t>(chunk_begin[n_long]) * tps;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total;
+       w += n_waves) {
+    const uint32_t chunk = static_cast<uint32_t>(w / tps);
+    const int t = static_cast<int>(w - static_cast<int64_t>(chunk) * tps);
+    // largest i with chunk_begin[i] <= chunk
+    uint32_t lo = 0, hi = n_long;
+    while (hi - lo > 1) {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (chunk_begin[mid] <= chunk) lo = mid; else hi = mid;
+    }
+    const uint32_t f = long_list[lo];
+    const uint32_t s0 = begin[f] + (chunk - chunk_begin[lo]) * kSegChunk;
+    const uint32_t s_end = begin[f + 1];
+    const uint32_t n = (s_end - s0) < static_cast<uint32_t>(kSegChunk) ? (s_end - s0) : kSegChunk;
+    const int pc = t * (kWave * VEC) + lane * VEC;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    accumulate_rows<PT, VEC, U>(P, s0, static_cast<int>(n), slice_w, pc, acc);
+    store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
+  }
+}
+
+// Long latents, step 2: out[f, slice] = sum of the latent's chunk partials, in chunk order.
+template <typename GT, int VEC, int U>
+__global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
+    const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
+    const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
+    void *__restrict__ out, int tps, int col0, int slice_w, int D) {
+  const int lane = lane_id();
+  const uint32_t n_long = *long_count;
+  const int64_t total = static_cast<int64_t>(n_long) * tps;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total;
+       w += n_waves) {
+    const uint32_t i = static_cast<uint32_t>(w / tps);
+    const int t = static_cast<int>(w - static_cast<int64_t>(i) * tps);
+    const int pc = t * (kWave * VEC) + lane * VEC;
+    const int d0 = col0 + pc;
+    const uint32_t c0 = chunk_begin[i], c1 = chunk_begin[i + 1];
+    float acc[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
+    accumulate_rows<float, VEC, U>(partial, c0, static_cast<int>(c1 - c0), slice_w, pc, acc);
+    if (d0 < D) store_vec<GT, VEC>(out, static_cast<int64_t>(long_list[i]) * D + d0, acc);
+  }
+}
+
+}  // namespace flexsae

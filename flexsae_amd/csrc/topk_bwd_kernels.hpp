@@ -31,55 +31,80 @@ __global__ void csr_count_kernel(const int64_t *__restrict__ indices, int64_t n_
   }
 }
 
-// In-place exclusive scan of begin[0..F) (holding counts on entry) by a single block;
-// begin[F] receives the total and cursor[0..F) a copy of the segment starts.
-constexpr int kScanThreads = 1024;
+// Exclusive scan of the per-latent counts in two launches.  Every block owns kScanBlockElems
+// consecutive latents: csr_scan_sums_kernel writes the block totals, csr_scan_apply_kernel
+// adds up the totals of the blocks before it (a few hundred values at most), scans its own
+// elements and writes begin[] and a copy for the fill cursor; the last block writes begin[F].
+constexpr int kScanThreads = 256;
 constexpr int kScanPerThread = 8;
-__global__ __launch_bounds__(kScanThreads) void csr_scan_kernel(uint32_t *__restrict__ begin,
-                                                                uint32_t *__restrict__ cursor,
-                                                                int64_t F) {
-  __shared__ uint32_t wave_tot[kScanThreads / kWave];
-  __shared__ uint32_t carry_s;
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wv = tid >> 6;
-  if (tid == 0) carry_s = 0;
+constexpr int kScanBlockElems = kScanThreads * kScanPerThread;
+
+__device__ __forceinline__ uint32_t block_sum_u32(uint32_t v, uint32_t *smem /*[kScanThreads/64]*/) {
+  // all threads receive the block total
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  const int wv = threadIdx.x >> 6;
   __syncthreads();
-  constexpr int64_t kChunk = static_cast<int64_t>(kScanThreads) * kScanPerThread;
-  for (int64_t base = 0; base < F; base += kChunk) {
-    uint32_t x[kScanPerThread];
-    uint32_t tsum = 0;
-    const int64_t i0 = base + static_cast<int64_t>(tid) * kScanPerThread;
+  if ((threadIdx.x & (kWave - 1)) == 0) smem[wv] = v;
+  __syncthreads();
+  uint32_t t = 0;
+  for (int w = 0; w < kScanThreads / kWave; ++w) t += smem[w];
+  return t;
+}
+
+__global__ __launch_bounds__(kScanThreads) void csr_scan_sums_kernel(const uint32_t *__restrict__ counts,
+                                                                     int64_t F,
+                                                                     uint32_t *__restrict__ block_sums) {
+  __shared__ uint32_t smem[kScanThreads / kWave];
+  const int64_t i0 = static_cast<int64_t>(blockIdx.x) * kScanBlockElems +
+                     static_cast<int64_t>(threadIdx.x) * kScanPerThread;
+  uint32_t tsum = 0;
 #pragma unroll
-    for (int i = 0; i < kScanPerThread; ++i) {
-      x[i] = (i0 + i < F) ? begin[i0 + i] : 0u;
-      tsum += x[i];
-    }
-    // inclusive scan of tsum across the wavefront
-    uint32_t inc = tsum;
+  for (int i = 0; i < kScanPerThread; ++i) tsum += (i0 + i < F) ? counts[i0 + i] : 0u;
+  const uint32_t tot = block_sum_u32(tsum, smem);
+  if (threadIdx.x == 0) block_sums[blockIdx.x] = tot;
+}
+
+__global__ __launch_bounds__(kScanThreads) void csr_scan_apply_kernel(uint32_t *__restrict__ begin,
+                                                                      uint32_t *__restrict__ cursor,
+                                                                      int64_t F,
+                                                                      const uint32_t *__restrict__ block_sums) {
+  __shared__ uint32_t smem[kScanThreads / kWave];
+  __shared__ uint32_t wave_tot[kScanThreads / kWave];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid >> 6;
+  // offset of this block = sum of the totals of all earlier blocks
+  uint32_t part = 0;
+  for (uint32_t j = tid; j < blockIdx.x; j += kScanThreads) part += block_sums[j];
+  const uint32_t block_off = block_sum_u32(part, smem);
+
+  const int64_t i0 = static_cast<int64_t>(blockIdx.x) * kScanBlockElems +
+                     static_cast<int64_t>(tid) * kScanPerThread;
+  uint32_t x[kScanPerThread];
+  uint32_t tsum = 0;
 #pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const uint32_t y = __shfl_up(inc, off, kWave);
-      if (lane >= off) inc += y;
-    }
-    if (lane == kWave - 1) wave_tot[wv] = inc;
-    __syncthreads();
-    uint32_t wave_off = 0;
-    for (int w = 0; w < wv; ++w) wave_off += wave_tot[w];
-    uint32_t run = carry_s + wave_off + (inc - tsum);
-#pragma unroll
-    for (int i = 0; i < kScanPerThread; ++i) {
-      if (i0 + i < F) {
-        begin[i0 + i] = run;
-        cursor[i0 + i] = run;
-      }
-      run += x[i];
-    }
-    __syncthreads();
-    if (tid == kScanThreads - 1) carry_s = run;
-    __syncthreads();
+  for (int i = 0; i < kScanPerThread; ++i) {
+    x[i] = (i0 + i < F) ? begin[i0 + i] : 0u;
+    tsum += x[i];
   }
-  if (tid == 0) begin[F] = carry_s;
+  uint32_t inc = tsum;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const uint32_t y = __shfl_up(inc, off, kWave);
+    if (lane >= off) inc += y;
+  }
+  if (lane == kWave - 1) wave_tot[wv] = inc;
+  __syncthreads();
+  uint32_t wave_off = 0;
+  for (int w = 0; w < wv; ++w) wave_off += wave_tot[w];
+  uint32_t run = block_off + wave_off + (inc - tsum);
+#pragma unroll
+  for (int i = 0; i < kScanPerThread; ++i) {
+    if (i0 + i < F) {
+      begin[i0 + i] = run;
+      cursor[i0 + i] = run;
+    }
+    run += x[i];
+  }
+  if (blockIdx.x == gridDim.x - 1 && tid == kScanThreads - 1) begin[F] = run;
 }
 
 __global__ void csr_fill_kernel(const int64_t *__restrict__ indices, int64_t n_pairs, int64_t F,
@@ -165,6 +190,14 @@ __global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__re
       }
     }
   }
+}
+
+// slot[map[s]] = s: position of every pair in the latent-major list.
+__global__ void csr_inverse_kernel(const uint32_t *__restrict__ map, int64_t n_pairs,
+                                   uint32_t *__restrict__ slot) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t s = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; s < n_pairs; s += stride)
+    slot[map[s]] = static_cast<uint32_t>(s);
 }
 
 // ---------------------------------------------------------------------------------
@@ -259,18 +292,33 @@ __global__ __launch_bounds__(256) void topk_bwd_kernel(
   if (active) store_vec<GT, VEC>(dW, f * D + d0, acc);
 }
 
-// dbias[d] += scale * sum_b resid[b, d]: grid (column blocks, row chunks).
-__global__ __launch_bounds__(256) void colsum_kernel(const float *__restrict__ resid,
-                                                     const float *__restrict__ grad_out, float coef,
-                                                     float *__restrict__ dbias, int64_t B, int D,
-                                                     int rows_per_block) {
-  const int d = blockIdx.x * blockDim.x + threadIdx.x;
-  if (d >= D) return;
-  const int64_t b0 = static_cast<int64_t>(blockIdx.y) * rows_per_block;
-  const int64_t b1 = (b0 + rows_per_block) < B ? (b0 + rows_per_block) : B;
+// Column sums of a row-major [rows, ld] fp32 matrix over `cols` columns, in two stages with a
+// fixed summation order (deterministic): stage 1 sums kColsumRows rows per block into
+// partial[chunk, cols]; stage 2 adds the chunks in order and writes
+// out[c] = scale * sum  with  scale = coef * (grad_out ? grad_out[0] : 1).
+constexpr int kColsumRows = 64;
+
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const float *__restrict__ x, int64_t rows,
+                                                             int64_t ld, int cols,
+                                                             float *__restrict__ partial) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * kColsumRows;
+  const int64_t r1 = (r0 + kColsumRows) < rows ? (r0 + kColsumRows) : rows;
   float s = 0.f;
-  for (int64_t b = b0; b < b1; ++b) s += resid[b * D + d];
-  unsafeAtomicAdd(dbias + d, s * coef * grad_out[0]);
+  for (int64_t r = r0; r < r1; ++r) s += x[r * ld + c];
+  partial[static_cast<int64_t>(blockIdx.y) * cols + c] = s;
+}
+
+__global__ __launch_bounds__(256) void colsum_final_kernel(const float *__restrict__ partial,
+                                                           int n_chunks, int cols,
+                                                           const float *__restrict__ grad_out, float coef,
+                                                           float *__restrict__ out) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  float s = 0.f;
+  for (int k = 0; k < n_chunks; ++k) s += partial[static_cast<int64_t>(k) * cols + c];
+  out[c] = s * coef * (grad_out ? grad_out[0] : 1.f);
 }
 
 __global__ void fill_f32_kernel(float *__restrict__ p, int64_t n) {

@@ -157,6 +157,18 @@ hier_fwd.register_fake(_fwd_fake)
 topk_fwd.register_fake(_fwd_fake)
 
 
+# Scratch the hierarchical backward may use for the per-pair contributions of one slice of D
+# columns.  More scratch = wider slices = fewer passes; 0 selects the atomic single-pass fallback.
+_hier_scratch_bytes = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
+
+
+def set_hier_scratch_bytes(nbytes: int) -> None:
+    """Upper bound on the scratch of the hierarchical backward (bytes).  0 = use the atomic
+    scatter fallback, which needs no scratch but an fp32 [F,D] accumulator."""
+    global _hier_scratch_bytes
+    _hier_scratch_bytes = int(nbytes)
+
+
 @torch.library.custom_op("flexsae_amd::hier_bwd", mutates_args=())
 def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
              resid: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
@@ -168,13 +180,24 @@ def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
     with torch.cuda.device(dev):
         g = _grad_scalar(grad_out, dev)
         shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
-        dW_acc = torch.empty((F, D), dtype=torch.float32, device=dev)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
-        rc = lib.flexsae_hier_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(resid),
-                                  _ptr(g), _ptr(dW_acc), _ptr(dvals), _ptr(dbias), 0,
-                                  _ptr(_flag_for(dev)), _stream())
-        _lib.check(rc, "flexsae_hier_bwd")
+        if _hier_scratch_bytes > 0:
+            p_size = 2 if weight.dtype == torch.bfloat16 else 4
+            slice_cols = max(1, _hier_scratch_bytes // (B * K * p_size))
+            ws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
+            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            dW = torch.empty_like(weight)
+            rc = lib.flexsae_hier_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(resid),
+                                      _ptr(g), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals), _ptr(dbias),
+                                      _ptr(workspace), ws_bytes, 0, _ptr(_flag_for(dev)), _stream())
+            _lib.check(rc, "flexsae_hier_bwd")
+            return dW, dvals, dbias
+        dW_acc = torch.empty((F, D), dtype=torch.float32, device=dev)
+        rc = lib.flexsae_hier_bwd_atomic(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals),
+                                         _ptr(resid), _ptr(g), _ptr(dW_acc), _ptr(dvals), _ptr(dbias), 0,
+                                         _ptr(_flag_for(dev)), _stream())
+        _lib.check(rc, "flexsae_hier_bwd_atomic")
         if weight.dtype == torch.float32:
             dW = dW_acc
         else:
@@ -205,9 +228,11 @@ def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
         dW = torch.empty_like(weight)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
+        bws_bytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(shape))
+        bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
         rc = lib.flexsae_topk_bwd(ctypes.byref(shape), _ptr(begin), _ptr(pair_map), _ptr(weight), _ptr(vals),
                                   _ptr(resid), _ptr(g), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals),
-                                  _ptr(dbias), 0, _stream())
+                                  _ptr(dbias), _ptr(bws), bws_bytes, 0, _stream())
         _lib.check(rc, "flexsae_topk_bwd")
     return dW, dvals, dbias
 

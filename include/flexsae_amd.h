@@ -93,17 +93,46 @@ int flexsae_topk_fwd(const flexsae_shape *shape, const int64_t *indices, const v
                      void *stream);
 
 /*
- * HierarchicalTopK backward: reverse sweep over K per row.
- * replaces: _hierarchical_sae_backward + hierarchical_sae_backward_kernel and the three
- *           mul_(grad) passes of HierarchicalSAELossFunction.backward
- *           (hierarchical_kernels.py:92-187, 230-270, 294-297)
+ * Bytes of workspace flexsae_hier_bwd needs to process `slice_cols` columns of D per pass
+ * (rounded up to whole 64*vec-column tiles, capped at D; slice_cols <= 0 asks for the minimum).
+ * The workspace holds the latent-major pair list, and per slice column one contribution per
+ * (b,k) pair (bf16 for bf16 weights, else fp32): about B*K*slice_cols*sizeof elements.
+ */
+size_t flexsae_hier_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slice_cols);
+
+/*
+ * HierarchicalTopK backward, two phases per slice of D columns:
+ *   sweep   : reverse walk over K per row; stores the per-pair contribution vals_k * S_k of the
+ *             slice into the workspace, accumulates dvals and dbias;
+ *   reduce  : latent-major segment reduction of those contributions (sorted pair list, fp32
+ *             accumulation, fixed order) writing dW once in `dW_dtype` -- no atomics on dW, the
+ *             result is deterministic, hot latents are split into 64-pair chunks.
+ * The number of passes is ceil(D / slice width); the slice width is the widest one the given
+ * workspace can hold (see flexsae_hier_bwd_workspace_bytes), so memory is the caller's choice.
+ * replaces: _hierarchical_sae_backward + hierarchical_sae_backward_kernel, the three
+ *           mul_(grad) passes of HierarchicalSAELossFunction.backward and the autograd engine's
+ *           cast of the fp32 gradient  (hierarchical_kernels.py:92-187, 230-270, 294-299)
  * in : resid from flexsae_hier_fwd; grad_out device scalar.
- * out: dW_acc[F,D] fp32 (scatter-add accumulator), dvals[B,K] fp32, dbias[D] fp32, all
- *      zero-filled here unless FLEXSAE_BWD_OUTPUTS_PREZEROED is set in `flags`.
+ * out: dW[F,D] in dW_dtype (every element written); dvals[B,K] fp32 (zero-filled here unless
+ *      FLEXSAE_BWD_OUTPUTS_PREZEROED); dbias[D] fp32 (written, fixed summation order).
  */
 int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
-                     const void *vals, const float *resid, const float *grad_out, float *dW_acc,
-                     float *dvals, float *dbias, int flags, int *status_flag, void *stream);
+                     const void *vals, const float *resid, const float *grad_out, void *dW,
+                     int dW_dtype, float *dvals, float *dbias, void *workspace,
+                     size_t workspace_bytes, int flags, int *status_flag, void *stream);
+
+/*
+ * HierarchicalTopK backward, single-pass fallback that needs no workspace: the same reverse
+ * sweep, scattering into an fp32 accumulator with atomics (as the reference kernel does).
+ * Slower (every contribution is a read-modify-write of dW in memory) and not bit-reproducible.
+ * replaces: same reference code as flexsae_hier_bwd.
+ * out: dW_acc[F,D] fp32, dvals[B,K] fp32, dbias[D] fp32, all zero-filled here unless
+ *      FLEXSAE_BWD_OUTPUTS_PREZEROED is set in `flags`.
+ */
+int flexsae_hier_bwd_atomic(const flexsae_shape *shape, const int64_t *indices, const void *weight,
+                            const void *vals, const float *resid, const float *grad_out,
+                            float *dW_acc, float *dvals, float *dbias, int flags, int *status_flag,
+                            void *stream);
 
 /* Bytes of workspace flexsae_csr_build needs. */
 size_t flexsae_csr_workspace_bytes(int64_t B, int64_t K, int64_t F);
@@ -127,13 +156,16 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
  *           (topk_kernels.py:97-137, 165-184, 220-223)
  * in : begin/map from flexsae_csr_build; resid from flexsae_topk_fwd; grad_out device scalar.
  * out: dW[F,D] written once in `dW_dtype` (every row, zeros for unused latents);
- *      dvals[B,K] fp32 and dbias[D] fp32 (zero-filled here unless
- *      FLEXSAE_BWD_OUTPUTS_PREZEROED).
+ *      dvals[B,K] fp32 (zero-filled here unless FLEXSAE_BWD_OUTPUTS_PREZEROED) and
+ *      dbias[D] fp32 (column sums in a fixed order: deterministic).
  */
 int flexsae_topk_bwd(const flexsae_shape *shape, const uint32_t *begin, const uint32_t *map,
                      const void *weight, const void *vals, const float *resid,
                      const float *grad_out, void *dW, int dW_dtype, float *dvals, float *dbias,
-                     int flags, void *stream);
+                     void *workspace, size_t workspace_bytes, int flags, void *stream);
+
+/* Bytes of workspace flexsae_topk_bwd needs (partial column sums for dbias). */
+size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *shape);
 
 /*
  * dst[n] (dtype) = src[n] (fp32), round-to-nearest-even.  Used to hand the fp32

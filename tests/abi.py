@@ -41,8 +41,25 @@ def forward(mode, indices, weight, vals, bias, target, flag=None):
     return rc, loss, resid
 
 
-def hier_backward(indices, weight, vals, resid, grad_out, flag=None, prezeroed=False):
-    """-> (rc, dW_acc fp32, dvals fp32, dbias fp32)."""
+def hier_backward(indices, weight, vals, resid, grad_out, flag=None, slice_cols=0, dw_dtype=torch.float32):
+    """Two-phase backward -> (rc, dW in dw_dtype, dvals fp32, dbias fp32); `slice_cols` sets the
+    workspace size (0 = the minimum, one tile per pass)."""
+    lib = _lib.load()
+    sh = shape_of(indices, weight, vals)
+    dev = weight.device
+    dW = torch.full((sh.F, sh.D), float("nan"), dtype=dw_dtype, device=dev)
+    dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
+    db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
+    g = torch.tensor([grad_out], dtype=torch.float32, device=dev)
+    nbytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    rc = lib.flexsae_hier_bwd(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(resid), ptr(g),
+                              ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, 0, ptr(flag), stream())
+    return rc, dW, dv, db
+
+
+def hier_backward_atomic(indices, weight, vals, resid, grad_out, flag=None, prezeroed=False):
+    """Atomic fallback -> (rc, dW_acc fp32, dvals fp32, dbias fp32)."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals)
     dev = weight.device
@@ -51,9 +68,9 @@ def hier_backward(indices, weight, vals, resid, grad_out, flag=None, prezeroed=F
     dv = torch.full((sh.B, sh.K), fill, dtype=torch.float32, device=dev)
     db = torch.full((sh.D,), fill, dtype=torch.float32, device=dev)
     g = torch.tensor([grad_out], dtype=torch.float32, device=dev)
-    rc = lib.flexsae_hier_bwd(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(resid), ptr(g),
-                              ptr(dW), ptr(dv), ptr(db), _lib.BWD_OUTPUTS_PREZEROED if prezeroed else 0,
-                              ptr(flag), stream())
+    rc = lib.flexsae_hier_bwd_atomic(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(resid),
+                                     ptr(g), ptr(dW), ptr(dv), ptr(db),
+                                     _lib.BWD_OUTPUTS_PREZEROED if prezeroed else 0, ptr(flag), stream())
     return rc, dW, dv, db
 
 
@@ -88,8 +105,10 @@ def topk_backward(indices, weight, vals, resid, grad_out, dw_dtype=None):
     dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
     db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
     g = torch.tensor([grad_out], dtype=torch.float32, device=dev)
+    nbytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     rc = lib.flexsae_topk_bwd(ctypes.byref(sh), ptr(begin), ptr(mp), ptr(weight), ptr(vals), ptr(resid),
-                              ptr(g), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), 0, stream())
+                              ptr(g), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, 0, stream())
     return rc, dW, dv, db
 
 

@@ -93,18 +93,39 @@ def test_backward_and_csr_reject_bad_arguments():
     lib = _lib.load()
     sh = _shape()
     ok = [FAKE] * 8
-    assert lib.flexsae_hier_bwd(ctypes.byref(_shape(D=0)), *ok, 0, NULL, NULL) == _lib.ERR_INVALID_ARGUMENT
+    atomic = lib.flexsae_hier_bwd_atomic
+    assert atomic(ctypes.byref(_shape(D=0)), *ok, 0, NULL, NULL) == _lib.ERR_INVALID_ARGUMENT
     for i in range(8):
         ptrs = [FAKE] * 8
         ptrs[i] = NULL
-        assert lib.flexsae_hier_bwd(ctypes.byref(sh), *ptrs, 0, NULL, NULL) == _lib.ERR_INVALID_ARGUMENT
+        assert atomic(ctypes.byref(sh), *ptrs, 0, NULL, NULL) == _lib.ERR_INVALID_ARGUMENT
+
+    def seg(shape, ptrs=None, ws=FAKE, ws_bytes=1 << 30, dw_dtype=0):
+        a = ptrs or [FAKE] * 8
+        return lib.flexsae_hier_bwd(ctypes.byref(shape), *a[:6], dw_dtype, a[6], a[7], ws, ws_bytes, 0, NULL, NULL)
+
+    assert seg(_shape(K=0)) == _lib.ERR_INVALID_ARGUMENT
+    assert seg(sh, dw_dtype=5) == _lib.ERR_INVALID_ARGUMENT
+    for i in range(8):
+        ptrs = [FAKE] * 8
+        ptrs[i] = NULL
+        assert seg(sh, ptrs) == _lib.ERR_INVALID_ARGUMENT
+    assert seg(sh, ws=NULL) == _lib.ERR_WORKSPACE
+    assert seg(sh, ws_bytes=64) == _lib.ERR_WORKSPACE
+    need_min = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), 0)
+    need_all = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), 1 << 30)
+    assert 0 < need_min <= need_all and need_min % 256 == 0
+    assert lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(_shape(B=-1)), 0) == 0
     assert lib.flexsae_csr_build(NULL, 4, 8, 16, FAKE, FAKE, FAKE, 1 << 20, NULL, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_csr_build(FAKE, 4, 8, 16, FAKE, FAKE, FAKE, 4, NULL, NULL) == _lib.ERR_WORKSPACE
     assert lib.flexsae_csr_build(FAKE, 1 << 20, 1 << 12, 16, FAKE, FAKE, FAKE, 1 << 20, NULL, NULL) == _lib.ERR_UNSUPPORTED
-    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 9, FAKE, FAKE, 0,
-                                NULL) == _lib.ERR_INVALID_ARGUMENT
-    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, NULL, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, 0,
-                                NULL) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 9, FAKE, FAKE, FAKE,
+                                1 << 20, 0, NULL) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, NULL, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, FAKE,
+                                1 << 20, 0, NULL) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, NULL,
+                                1 << 20, 0, NULL) == _lib.ERR_WORKSPACE
+    assert lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh)) >= 64 * 4
     assert lib.flexsae_cast_from_f32(NULL, 1, FAKE, 10, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_cast_from_f32(FAKE, 1, FAKE, -1, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_cast_from_f32(FAKE, 1, FAKE, 0, NULL) == _lib.OK
