@@ -4,6 +4,7 @@
 
 #include "common.hpp"
 #include "fwd_kernels.hpp"
+#include "csr_kernels.hpp"
 #include "hier_bwd_kernels.hpp"
 #include "segment_kernels.hpp"
 #include "topk_bwd_kernels.hpp"
@@ -180,49 +181,6 @@ void launch_hier_bwd_t(const flexsae_shape *s, const int64_t *indices, const voi
 void zero_f32(float *p, int64_t n, hipStream_t st) {
   hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_for(ceil_div(n, 4), 256, 1 << 16)), dim3(256), 0, st,
                      p, n);
-}
-
-template <typename WT, typename GT>
-void launch_topk_bwd_t(const flexsae_shape *s, const uint32_t *begin, const uint32_t *map,
-                       const void *weight, const void *vals, const float *resid,
-                       const float *grad_out, float coef, void *dW, float *dvals, int vec,
-                       hipStream_t st) {
-  const int K = static_cast<int>(s->K), D = static_cast<int>(s->D);
-  const int ntiles = static_cast<int>(ceil_div(D, static_cast<int64_t>(kWave) * vec));
-  const int64_t n_items = s->F * ntiles;
-  const unsigned grid = static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock));
-#define FLEXSAE_LAUNCH_TB(VV)                                                                     \
-  hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, VV, 4, true>), dim3(grid), dim3(kBlock), 0, st,     \
-                     begin, map, weight, vals, s->vals_dtype, resid, grad_out, coef, dW, dvals,   \
-                     n_items, ntiles, s->F, K, D)
-  if (vec == 4) {
-    FLEXSAE_LAUNCH_TB(4);
-  } else if (vec == 2) {
-    FLEXSAE_LAUNCH_TB(2);
-  } else {
-    FLEXSAE_LAUNCH_TB(1);
-  }
-#undef FLEXSAE_LAUNCH_TB
-}
-
-template <typename WT>
-void launch_topk_bwd_g(const flexsae_shape *s, const uint32_t *begin, const uint32_t *map,
-                       const void *weight, const void *vals, const float *resid,
-                       const float *grad_out, float coef, void *dW, int dW_dtype, float *dvals,
-                       int vec, hipStream_t st) {
-  switch (dW_dtype) {
-    case FLEXSAE_F32:
-      launch_topk_bwd_t<WT, float>(s, begin, map, weight, vals, resid, grad_out, coef, dW, dvals,
-                                   vec, st);
-      break;
-    case FLEXSAE_BF16:
-      launch_topk_bwd_t<WT, bf16_t>(s, begin, map, weight, vals, resid, grad_out, coef, dW, dvals,
-                                    vec, st);
-      break;
-    default:
-      launch_topk_bwd_t<WT, f16_t>(s, begin, map, weight, vals, resid, grad_out, coef, dW, dvals,
-                                   vec, st);
-  }
 }
 
 // Scratch of the pair-list construction, carved out of one workspace:
@@ -411,6 +369,107 @@ void launch_hier_slices_w(const flexsae_shape *s, const HierBwdPlan &pl, int64_t
   }
 }
 
+// ---- TopK backward: workspace plan and slice loop ---------------------------------------
+
+struct TopkBwdPlan {
+  int vec, tile;
+  int64_t d_pad;
+  size_t n_pairs, n_partial_rows;
+  size_t off_colsum, off_long_count, off_long_list, off_chunk, off_partial, fixed_bytes;
+};
+
+TopkBwdPlan plan_topk_bwd(const flexsae_shape *s) {
+  TopkBwdPlan p;
+  p.vec = (s->D % 4 == 0) ? 4 : (s->D % 2 == 0) ? 2 : 1;
+  p.tile = kWave * p.vec;
+  p.d_pad = ceil_div(s->D, p.tile) * p.tile;
+  p.n_pairs = static_cast<size_t>(s->B) * static_cast<size_t>(s->K);
+  p.n_partial_rows = p.n_pairs / kSegChunk + p.n_pairs / 65 + 2;
+  size_t off = 0;
+  p.off_colsum = off;
+  off += round_up(static_cast<size_t>(ceil_div(s->B, kColsumRows)) * static_cast<size_t>(s->D) * 4, kAlign);
+  p.off_long_count = off;
+  off += kAlign;
+  p.off_long_list = off;
+  off += round_up((p.n_pairs / 65 + 1) * 4, kAlign);
+  p.off_chunk = off;
+  off += round_up((p.n_pairs / 65 + 2) * 4, kAlign);
+  p.off_partial = off;
+  p.fixed_bytes = off;
+  return p;
+}
+
+size_t topk_bwd_bytes(const TopkBwdPlan &p, int64_t slice_w) {
+  return p.fixed_bytes + round_up(p.n_partial_rows * static_cast<size_t>(slice_w) * 4, kAlign);
+}
+
+template <typename WT, typename GT, int VEC>
+void launch_topk_slices(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t slice_w,
+                        const uint32_t *begin, const uint32_t *map, const void *weight,
+                        const void *vals, const float *resid, const float *grad_out, float coef,
+                        void *dW, float *dvals, uint8_t *ws, hipStream_t st) {
+  const uint32_t *long_count = reinterpret_cast<const uint32_t *>(ws + pl.off_long_count);
+  const uint32_t *long_list = reinterpret_cast<const uint32_t *>(ws + pl.off_long_list);
+  const uint32_t *chunk_begin = reinterpret_cast<const uint32_t *>(ws + pl.off_chunk);
+  float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
+  const int K = static_cast<int>(s->K), D = static_cast<int>(s->D), sw = static_cast<int>(slice_w);
+  for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
+    const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
+    const int tps = static_cast<int>(cols / pl.tile);
+    const int64_t n_items = s->F * tps;
+    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, VEC, 4>),
+                       dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
+                       begin, map, weight, vals, s->vals_dtype, resid, grad_out, coef, dW, dvals, n_items,
+                       static_cast<int>(col0), s->F, K, D);
+    hipLaunchKernelGGL((topk_bwd_long_kernel<WT, VEC, 4>), dim3(1024), dim3(kBlock), 0, st, begin, map,
+                       long_count, long_list, chunk_begin, weight, vals, s->vals_dtype, resid, grad_out,
+                       coef, dvals, partial, tps, static_cast<int>(col0), sw, K, D);
+    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
+                       long_count, long_list, chunk_begin, partial, dW, tps, static_cast<int>(col0), sw,
+                       D);
+  }
+}
+
+template <typename WT, int VEC>
+void launch_topk_slices_g(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t slice_w,
+                          const uint32_t *begin, const uint32_t *map, const void *weight,
+                          const void *vals, const float *resid, const float *grad_out, float coef,
+                          void *dW, int dW_dtype, float *dvals, uint8_t *ws, hipStream_t st) {
+  switch (dW_dtype) {
+    case FLEXSAE_F32:
+      launch_topk_slices<WT, float, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef,
+                                         dW, dvals, ws, st);
+      break;
+    case FLEXSAE_BF16:
+      launch_topk_slices<WT, bf16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef,
+                                          dW, dvals, ws, st);
+      break;
+    default:
+      launch_topk_slices<WT, f16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef,
+                                         dW, dvals, ws, st);
+  }
+}
+
+template <int VEC>
+void launch_topk_slices_w(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t slice_w,
+                          const uint32_t *begin, const uint32_t *map, const void *weight,
+                          const void *vals, const float *resid, const float *grad_out, float coef,
+                          void *dW, int dW_dtype, float *dvals, uint8_t *ws, hipStream_t st) {
+  switch (s->weight_dtype) {
+    case FLEXSAE_F32:
+      launch_topk_slices_g<float, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW,
+                                       dW_dtype, dvals, ws, st);
+      break;
+    case FLEXSAE_BF16:
+      launch_topk_slices_g<bf16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW,
+                                        dW_dtype, dvals, ws, st);
+      break;
+    default:
+      launch_topk_slices_g<f16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW,
+                                       dW_dtype, dvals, ws, st);
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -570,9 +629,12 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
   return launch_status();
 }
 
-size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *s) {
+size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_cols) {
   if (check_shape(s) != FLEXSAE_OK) return 0;
-  return round_up(static_cast<size_t>(ceil_div(s->B, kColsumRows)) * static_cast<size_t>(s->D) * 4, kAlign);
+  const TopkBwdPlan pl = plan_topk_bwd(s);
+  int64_t sw = slice_cols <= 0 ? pl.tile : ceil_div(slice_cols, pl.tile) * pl.tile;
+  if (sw > pl.d_pad) sw = pl.d_pad;
+  return topk_bwd_bytes(pl, sw);
 }
 
 int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32_t *map,
@@ -584,40 +646,43 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
   if (!begin || !map || !weight || !vals || !resid || !grad_out || !dW || !dvals || !dbias ||
       !valid_dtype(dW_dtype))
     return FLEXSAE_ERR_INVALID_ARGUMENT;
-  if (!aligned(begin, 4) || !aligned(map, 4) || !aligned(weight, dtype_size(s->weight_dtype)) ||
-      !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, 4) || !aligned(grad_out, 4) ||
-      !aligned(dW, dtype_size(dW_dtype)) || !aligned(dvals, 16) || !aligned(dbias, 4))
+  const TopkBwdPlan pl = plan_topk_bwd(s);
+  if (!aligned(begin, 4) || !aligned(map, 4) || !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
+      !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.vec * 4) || !aligned(grad_out, 4) ||
+      !aligned(dW, pl.vec * dtype_size(dW_dtype)) || !aligned(dvals, 16) || !aligned(dbias, 4))
     return FLEXSAE_ERR_ALIGNMENT;
-  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < flexsae_topk_bwd_workspace_bytes(s))
+  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < topk_bwd_bytes(pl, pl.tile))
     return FLEXSAE_ERR_WORKSPACE;
+  int64_t slice_w = pl.tile;
+  while (slice_w + pl.tile <= pl.d_pad && topk_bwd_bytes(pl, slice_w + pl.tile) <= workspace_bytes)
+    slice_w += pl.tile;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
   if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) zero_f32(dvals, s->B * s->K, st);
+  // latents with more than 64 pairs and their chunk table
+  uint32_t *long_count = reinterpret_cast<uint32_t *>(ws + pl.off_long_count);
+  uint32_t *long_list = reinterpret_cast<uint32_t *>(ws + pl.off_long_list);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, long_count, static_cast<int64_t>(1), 0u);
+  hipLaunchKernelGGL(seg_find_long_kernel, dim3(grid_for(s->F, 256, 2048)), dim3(256), 0, st, begin, s->F,
+                     long_count, long_list);
+  hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, long_count, long_list,
+                     reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
   const float coef =
       static_cast<float>(2.0 / (static_cast<double>(s->B) * static_cast<double>(s->D)));
-  // vector width: resid rows are read as fp32 vectors, weight/dW rows in their own types
-  int vec = 4;
-  while (vec > 1 && (s->D % vec != 0 || !aligned(resid, vec * 4) ||
-                     !aligned(weight, vec * dtype_size(s->weight_dtype)) ||
-                     !aligned(dW, vec * dtype_size(dW_dtype))))
-    vec >>= 1;
-  while (vec > 1 && s->D < static_cast<int64_t>(kWave) * vec && s->D % (vec / 2) == 0) vec >>= 1;
-  switch (s->weight_dtype) {
-    case FLEXSAE_F32:
-      launch_topk_bwd_g<float>(s, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                               dvals, vec, st);
-      break;
-    case FLEXSAE_BF16:
-      launch_topk_bwd_g<bf16_t>(s, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                                dvals, vec, st);
-      break;
-    default:
-      launch_topk_bwd_g<f16_t>(s, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                               dvals, vec, st);
+  if (pl.vec == 4) {
+    launch_topk_slices_w<4>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
+                            dvals, ws, st);
+  } else if (pl.vec == 2) {
+    launch_topk_slices_w<2>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
+                            dvals, ws, st);
+  } else {
+    launch_topk_slices_w<1>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
+                            dvals, ws, st);
   }
   rc = launch_status();
   if (rc != FLEXSAE_OK) return rc;
   // dbias = coef * grad_out * column sums of resid, in a fixed order
-  float *colsum_part = static_cast<float *>(workspace);
+  float *colsum_part = reinterpret_cast<float *>(ws + pl.off_colsum);
   const int n_chunks = static_cast<int>(ceil_div(s->B, kColsumRows));
   const int D = static_cast<int>(s->D);
   hipLaunchKernelGGL(colsum_partial_kernel,

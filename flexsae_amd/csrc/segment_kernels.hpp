@@ -56,6 +56,17 @@ __global__ __launch_bounds__(256) void seg_reduce_short_kernel(
   }
 }
 
+// long_list[0..*long_count) = latents with more than kSegChunk pairs (any order);
+// *long_count must be zero on entry.
+__global__ void seg_find_long_kernel(const uint32_t *__restrict__ begin, int64_t F,
+                                     uint32_t *__restrict__ long_count,
+                                     uint32_t *__restrict__ long_list) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t f = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; f < F; f += stride)
+    if (begin[f + 1] - begin[f] > static_cast<uint32_t>(kSegChunk))
+      long_list[atomicAdd(long_count, 1u)] = static_cast<uint32_t>(f);
+}
+
 // chunk_begin[i] = number of chunks of the long latents before long_list[i]
 // (chunk_begin[n_long] = total); single block.
 __global__ __launch_bounds__(1024) void seg_chunk_table_kernel(const uint32_t *__restrict__ begin,

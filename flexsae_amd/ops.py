@@ -228,7 +228,9 @@ def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
         dW = torch.empty_like(weight)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
-        bws_bytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(shape))
+        # the slice width only sizes the partial sums of hot latents: 64 MiB of them is plenty
+        slice_cols = max(1, (64 << 20) // max(1, (B * K // 32) * 4))
+        bws_bytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
         bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
         rc = lib.flexsae_topk_bwd(ctypes.byref(shape), _ptr(begin), _ptr(pair_map), _ptr(weight), _ptr(vals),
                                   _ptr(resid), _ptr(g), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals),

@@ -164,8 +164,13 @@ int flexsae_topk_bwd(const flexsae_shape *shape, const uint32_t *begin, const ui
                      const float *grad_out, void *dW, int dW_dtype, float *dvals, float *dbias,
                      void *workspace, size_t workspace_bytes, int flags, void *stream);
 
-/* Bytes of workspace flexsae_topk_bwd needs (partial column sums for dbias). */
-size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *shape);
+/*
+ * Bytes of workspace flexsae_topk_bwd needs to process `slice_cols` columns of D per pass
+ * (rounded to whole tiles, capped at D; <= 0 asks for the minimum).  The slice width only
+ * sizes the fp32 partial sums of latents with more than 64 pairs (hot latents are cut into
+ * 64-pair chunks that are reduced by separate wavefronts and then combined in a fixed order).
+ */
+size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slice_cols);
 
 /*
  * dst[n] (dtype) = src[n] (fp32), round-to-nearest-even.  Used to hand the fp32

@@ -92,7 +92,7 @@ def widen_u32(t):
     return t.to(torch.int64) & 0xFFFFFFFF
 
 
-def topk_backward(indices, weight, vals, resid, grad_out, dw_dtype=None):
+def topk_backward(indices, weight, vals, resid, grad_out, dw_dtype=None, slice_cols=0):
     """-> (rc, dW in dw_dtype, dvals fp32, dbias fp32); builds the pair list first."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals)
@@ -105,7 +105,7 @@ def topk_backward(indices, weight, vals, resid, grad_out, dw_dtype=None):
     dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
     db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
     g = torch.tensor([grad_out], dtype=torch.float32, device=dev)
-    nbytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh))
+    nbytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     rc = lib.flexsae_topk_bwd(ctypes.byref(sh), ptr(begin), ptr(mp), ptr(weight), ptr(vals), ptr(resid),
                               ptr(g), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, 0, stream())

@@ -125,7 +125,9 @@ def test_backward_and_csr_reject_bad_arguments():
                                 1 << 20, 0, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, NULL,
                                 1 << 20, 0, NULL) == _lib.ERR_WORKSPACE
-    assert lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh)) >= 64 * 4
+    assert lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh), 0) >= 64 * 4
+    assert (lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh), 1 << 30)
+            >= lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh), 0))
     assert lib.flexsae_cast_from_f32(NULL, 1, FAKE, 10, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_cast_from_f32(FAKE, 1, FAKE, -1, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_cast_from_f32(FAKE, 1, FAKE, 0, NULL) == _lib.OK

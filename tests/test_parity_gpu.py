@@ -222,6 +222,45 @@ def test_hier_slice_width_does_not_change_the_result(shape, dtype):
         assert rel_err(dv.cpu(), rv) < 1e-4 and rel_err(db.cpu(), rb) < 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("shape", [(64, 32, 224, 1024), (33, 12, 17, 2304), (96, 130, 9, 200), (256, 64, 3, 70)])
+def test_topk_slice_width_does_not_change_the_result(shape, dtype):
+    """Same for the TopK backward: hot latents (F tiny) go through 64-pair chunks whose partial
+    sums live in a slice-wide workspace; any slice width must give bit-identical dW."""
+    B, K, F, D = shape
+    _announce("topk slices", shape, dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=32)
+    idx, W, v, b, t = _to_dev(args)
+    rc, loss, resid = abi.forward("topk", idx, W, v, b, t)
+    assert rc == 0
+    outs = []
+    for cols in (0, 512, 1 << 20):
+        rc, dW, dv, db = abi.topk_backward(idx, W, v, resid, 0.9, dw_dtype=torch.float32, slice_cols=cols)
+        assert rc == 0
+        outs.append((dW, dv, db))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[1][0], outs[2][0])
+    assert torch.equal(outs[0][2], outs[1][2])  # dbias: fixed-order column sums
+    L, rW, rv, rb = oracle.loss_grads(oracle.TOPK, *args, grad_out=0.9)
+    assert rel_err(outs[0][0].cpu(), rW) < 1e-4
+    for _, dv, db in outs:
+        assert rel_err(dv.cpu(), rv) < 1e-4 and rel_err(db.cpu(), rb) < 1e-4
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_skewed_latents(mode, dtype):
+    """Zipf-distributed per-row-unique indices with vals sorted descending (the shape of the
+    skewed BASELINE configuration, scaled down): a few latents appear in almost every row."""
+    B, K, F, D = 512, 16, 4096, 512
+    _announce("zipf", mode, dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=77, zipf_s=1.1, sort_vals=True, w_std=0.02)
+    counts = torch.bincount(args[0].flatten(), minlength=F)
+    assert counts.max() > 300  # hot latents really are hot
+    got = _run_op(mode, args, 1.0)
+    _check_against_oracle(mode, args, dtype, 1.0, got, ref_tols=False)
+
+
 def test_hier_dw_is_reproducible_bit_for_bit():
     args = _to_dev(make_inputs(96, 32, 64, 1536, seed=9))  # F small: long groups, many collisions
     idx, W, v, b, t = args
