@@ -215,7 +215,7 @@ def main():
     topk_peak = torch.cuda.max_memory_allocated() - base_mem
     Wp.grad = vp.grad = bp.grad = None
 
-    # ---- dominant kernels alone, HIP events on the launch stream -------------------------
+    # ---- kernels alone, HIP events on the launch stream -----------------------------------
     DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
     sh = _lib.Shape(B, K, F, D, DT[dtype], DT[dtype], DT[dtype], DT[dtype])
     p = lambda x: ctypes.c_void_p(x.data_ptr())
@@ -228,39 +228,76 @@ def main():
     dvals = torch.empty(B, K, dtype=torch.float32, device=dev)
     dbias = torch.empty(D, dtype=torch.float32, device=dev)
     dW = torch.empty(F, D, dtype=dtype, device=dev)
+    p_size = 2 if dtype == torch.bfloat16 else 4
     scratch = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
-    slice_cols = max(1, scratch // (B * K * (2 if dtype == torch.bfloat16 else 4)))
+    slice_cols = max(1, scratch // (B * K * p_size))
     bws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
     bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
+    tile = 64 * (4 if D % 4 == 0 else 2 if D % 2 == 0 else 1)
+    d_pad = -(-D // tile) * tile
+    slice_w = min(d_pad, max(tile, -(-slice_cols // tile) * tile))
+    n_slices = -(-D // slice_w)
 
     def fwd_launch():
         _lib.check(lib.flexsae_hier_fwd(ctypes.byref(sh), p(idx), p(W), p(v), p(b), p(t), p(loss), p(resid), p(ws),
                                         ws_bytes, None, st()), "flexsae_hier_fwd")
 
-    def bwd_launch():
+    def bwd_launch(flags=0):
         _lib.check(lib.flexsae_hier_bwd(ctypes.byref(sh), p(idx), p(W), p(v), p(resid), p(g1), p(dW), DT[dtype],
-                                        p(dvals), p(dbias), p(bws), bws_bytes, 0, None, st()), "flexsae_hier_bwd")
+                                        p(dvals), p(dbias), p(bws), bws_bytes, flags, None, st()),
+                   "flexsae_hier_bwd")
 
+    PRE, REUSE, SWEEP, REDUCE = 1, 2, 4, 8
     fwd_k_ms = time_kernel_events(torch, lambda: None, fwd_launch, args.steps, args.warmup)
-    bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
+    if scratch > 0:
+        bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
+        # the pair list is in the workspace now: time the two phases alone (n_slices launches each)
+        sweep_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(PRE | REUSE | SWEEP), args.steps, 1)
+        reduce_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(PRE | REUSE | REDUCE), args.steps, 1)
+        sweep_name = "hier_sweep_kernel"
+    else:
+        # scratch budget 0 selects the single-pass atomic fallback (one launch, fp32 accumulator)
+        dW_acc = torch.empty(F, D, dtype=torch.float32, device=dev)
+
+        def atomic_launch():
+            _lib.check(lib.flexsae_hier_bwd_atomic(ctypes.byref(sh), p(idx), p(W), p(v), p(resid), p(g1), p(dW_acc),
+                                                   p(dvals), p(dbias), PRE, None, st()), "flexsae_hier_bwd_atomic")
+
+        def atomic_prepare():
+            dW_acc.zero_()
+            dvals.zero_()
+            dbias.zero_()
+
+        bwd_k_ms = time_kernel_events(torch, atomic_prepare, atomic_launch, args.steps, args.warmup)
+        sweep_ms, reduce_ms, n_slices, sweep_name = bwd_k_ms, 0.0, 1, "hier_bwd_kernel (atomic fallback)"
+        del dW_acc
     del dW, bws
 
     def gbps(nbytes, ms):
         return nbytes / (ms * 1e-3) / 1e9
 
-    dominant = "flexsae_hier_bwd (pair list + sweep + segment reduce)" if bwd_k_ms >= fwd_k_ms else "sae_fwd_kernel(hier)"
-    dom_bytes = abytes["hier_bwd_kernel"] if bwd_k_ms >= fwd_k_ms else abytes["fwd_kernel"]
-    dom_ms = max(bwd_k_ms, fwd_k_ms)
+    # algorithmic bytes of ONE sweep launch: its share of the gathered rows, indices/vals/slots,
+    # and the residual slice (the staged contributions are traffic, not algorithmic bytes)
+    sweep_launch_bytes = (B * K * D * es + B * K * (8 + es + 4) * n_slices + B * D * 4) / n_slices
+    sweep_launch_ms = sweep_ms / n_slices
+    traffic = None
+    traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    if os.path.exists(traffic_file) and not args.shape:
+        with open(traffic_file) as fh:
+            rec = json.load(fh).get(f"{args.workload}:{scratch >> 20}")
+        if rec:
+            traffic = rec["hier_sweep_kernel_bytes_per_launch"]
     roofline = {
         "bound": "hbm",
-        "kernel": dominant,
-        "achieved": round(gbps(dom_bytes, dom_ms), 1),
+        "kernel": sweep_name,
+        "achieved": round(gbps(sweep_launch_bytes, sweep_launch_ms), 1),
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
-        "frac": round(gbps(dom_bytes, dom_ms) / HBM_PEAK_GBPS, 4),
-        "traffic": None,
-        "algorithmic_bytes": dom_bytes,
-        "avg_launch_ms": round(dom_ms, 4),
+        "frac": round(gbps(sweep_launch_bytes, sweep_launch_ms) / HBM_PEAK_GBPS, 4),
+        "traffic": traffic,
+        "algorithmic_bytes_per_launch": int(sweep_launch_bytes),
+        "avg_launch_ms": round(sweep_launch_ms, 4),
+        "launches_per_step": n_slices,
     }
 
     out = {
@@ -277,16 +314,22 @@ def main():
         "dtype": "f32 arithmetic on %s storage" % dt_name,
         "data": "synthetic",
         "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
-                               f"indices {dist}", "B": B, "K": K, "F": F, "D": D},
+                               f"indices {dist}", "B": B, "K": K, "F": F, "D": D,
+                   "hier_scratch_mb": scratch >> 20},
         "roofline": roofline,
         "step_hbm": {"algorithmic_bytes": abytes["hier_step"],
                      "achieved_GBps": round(gbps(abytes["hier_step"], hier_ms), 1),
                      "frac_of_peak": round(gbps(abytes["hier_step"], hier_ms) / HBM_PEAK_GBPS, 4)},
         "kernels": {
-            "sae_fwd_kernel(hier)": {"ms": round(fwd_k_ms, 4), "algorithmic_bytes": abytes["fwd_kernel"],
-                                     "GBps": round(gbps(abytes["fwd_kernel"], fwd_k_ms), 1)},
-            "flexsae_hier_bwd": {"ms": round(bwd_k_ms, 4), "algorithmic_bytes": abytes["hier_bwd_kernel"],
-                                "GBps": round(gbps(abytes["hier_bwd_kernel"], bwd_k_ms), 1)},
+            "flexsae_hier_fwd (sae_fwd_kernel + loss_finalize)": {
+                "ms": round(fwd_k_ms, 4), "algorithmic_bytes": abytes["fwd_kernel"],
+                "GBps": round(gbps(abytes["fwd_kernel"], fwd_k_ms), 1),
+                "frac_of_peak": round(gbps(abytes["fwd_kernel"], fwd_k_ms) / HBM_PEAK_GBPS, 4)},
+            "flexsae_hier_bwd (pair list + sweep + reduce)": {
+                "ms": round(bwd_k_ms, 4), "algorithmic_bytes": abytes["hier_bwd_kernel"],
+                "GBps": round(gbps(abytes["hier_bwd_kernel"], bwd_k_ms), 1)},
+            "%s x%d" % (sweep_name, n_slices): {"ms": round(sweep_ms, 4)},
+            "segment reduction x%d" % n_slices: {"ms": round(reduce_ms, 4)},
         },
         "topk": {"ms_per_step": round(topk_ms, 4), "algorithmic_bytes": abytes["topk_step"],
                  "achieved_GBps": round(gbps(abytes["topk_step"], topk_ms), 1)},

@@ -214,7 +214,15 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const float *__rest
   const int64_t r0 = static_cast<int64_t>(blockIdx.y) * kColsumRows;
   const int64_t r1 = (r0 + kColsumRows) < rows ? (r0 + kColsumRows) : rows;
   float s = 0.f;
-  for (int64_t r = r0; r < r1; ++r) s += x[r * ld + c];
+  int64_t r = r0;
+  for (; r + 8 <= r1; r += 8) {  // eight independent loads in flight
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = x[(r + u) * ld + c];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
+  }
+  for (; r < r1; ++r) s += x[r * ld + c];
   partial[static_cast<int64_t>(blockIdx.y) * cols + c] = s;
 }
 
@@ -225,7 +233,15 @@ __global__ __launch_bounds__(256) void colsum_final_kernel(const float *__restri
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= cols) return;
   float s = 0.f;
-  for (int k = 0; k < n_chunks; ++k) s += partial[static_cast<int64_t>(k) * cols + c];
+  int k = 0;
+  for (; k + 8 <= n_chunks; k += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = partial[static_cast<int64_t>(k + u) * cols + c];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
+  }
+  for (; k < n_chunks; ++k) s += partial[static_cast<int64_t>(k) * cols + c];
   out[c] = s * coef * (grad_out ? grad_out[0] : 1.f);
 }
 

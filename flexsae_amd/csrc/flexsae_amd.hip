@@ -289,7 +289,10 @@ template <typename WT, typename PT, typename GT, int VEC>
 void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t slice_w,
                         const int64_t *indices, const void *weight, const void *vals,
                         const float *resid, const float *grad_out, float coef, void *dW,
-                        float *dvals, float *dbias, uint8_t *ws, int *status_flag, hipStream_t st) {
+                        float *dvals, float *dbias, uint8_t *ws, int flags, int *status_flag,
+                        hipStream_t st) {
+  const bool do_sweep = !(flags & FLEXSAE_BWD_REDUCE_ONLY);
+  const bool do_reduce = !(flags & FLEXSAE_BWD_SWEEP_ONLY);
   const uint32_t *begin = reinterpret_cast<const uint32_t *>(ws + pl.off_begin);
   const uint32_t *slot = reinterpret_cast<const uint32_t *>(ws + pl.off_slot);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
@@ -306,10 +309,13 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
     const int64_t sweep_items = s->B * tps;
-    hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, 8>),
-                       dim3(static_cast<unsigned>(ceil_div(sweep_items, kWavesPerBlock))), dim3(kBlock),
-                       0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dvals,
-                       s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F, D);
+    if (do_sweep)
+      hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, 8>),
+                         dim3(static_cast<unsigned>(ceil_div(sweep_items, kWavesPerBlock))), dim3(kBlock),
+                         0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dvals,
+                         s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F,
+                         D);
+    if (!do_reduce) continue;
     hipLaunchKernelGGL((seg_reduce_short_kernel<PT, GT, VEC, 8>),
                        dim3(static_cast<unsigned>(ceil_div(s->F, kWavesPerBlock))), dim3(kBlock), 0, st,
                        begin, P, dW, s->F, tps, static_cast<int>(col0), sw, D);
@@ -319,6 +325,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                        sc.long_count, sc.long_list, chunk_begin, partial, dW, tps,
                        static_cast<int>(col0), sw, D);
   }
+  if (!do_sweep || !do_reduce) return;
   // dbias = column sums of s_final over the rows, in a fixed order
   hipLaunchKernelGGL(colsum_partial_kernel,
                      dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
@@ -331,20 +338,20 @@ template <typename WT, typename PT, int VEC>
 void launch_hier_slices_g(const flexsae_shape *s, const HierBwdPlan &pl, int64_t slice_w,
                           const int64_t *indices, const void *weight, const void *vals,
                           const float *resid, const float *grad_out, float coef, void *dW,
-                          int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int *status_flag,
-                          hipStream_t st) {
+                          int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int flags,
+                          int *status_flag, hipStream_t st) {
   switch (dW_dtype) {
     case FLEXSAE_F32:
       launch_hier_slices<WT, PT, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                             coef, dW, dvals, dbias, ws, status_flag, st);
+                                             coef, dW, dvals, dbias, ws, flags, status_flag, st);
       break;
     case FLEXSAE_BF16:
       launch_hier_slices<WT, PT, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dvals, dbias, ws, status_flag, st);
+                                              coef, dW, dvals, dbias, ws, flags, status_flag, st);
       break;
     default:
       launch_hier_slices<WT, PT, f16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                             coef, dW, dvals, dbias, ws, status_flag, st);
+                                             coef, dW, dvals, dbias, ws, flags, status_flag, st);
   }
 }
 
@@ -352,20 +359,20 @@ template <int VEC>
 void launch_hier_slices_w(const flexsae_shape *s, const HierBwdPlan &pl, int64_t slice_w,
                           const int64_t *indices, const void *weight, const void *vals,
                           const float *resid, const float *grad_out, float coef, void *dW,
-                          int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int *status_flag,
-                          hipStream_t st) {
+                          int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int flags,
+                          int *status_flag, hipStream_t st) {
   switch (s->weight_dtype) {
     case FLEXSAE_F32:
       launch_hier_slices_g<float, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dW_dtype, dvals, dbias, ws, status_flag, st);
+                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st);
       break;
     case FLEXSAE_BF16:
       launch_hier_slices_g<bf16_t, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                                coef, dW, dW_dtype, dvals, dbias, ws, status_flag, st);
+                                                coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st);
       break;
     default:
       launch_hier_slices_g<f16_t, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dW_dtype, dvals, dbias, ws, status_flag, st);
+                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st);
   }
 }
 
@@ -588,22 +595,24 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
-  csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
-  hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
-                     s->B * s->K, reinterpret_cast<uint32_t *>(ws + pl.off_slot));
-  hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
-                     sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+  if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
+    csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
+    hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
+                       s->B * s->K, reinterpret_cast<uint32_t *>(ws + pl.off_slot));
+    hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
+                       sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+  }
   const float coef = static_cast<float>(
       2.0 / (static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D)));
   if (pl.vec == 4) {
     launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                            dvals, dbias, ws, status_flag, st);
+                            dvals, dbias, ws, flags, status_flag, st);
   } else if (pl.vec == 2) {
     launch_hier_slices_w<2>(s, pl, slice_w, indices, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                            dvals, dbias, ws, status_flag, st);
+                            dvals, dbias, ws, flags, status_flag, st);
   } else {
     launch_hier_slices_w<1>(s, pl, slice_w, indices, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                            dvals, dbias, ws, status_flag, st);
+                            dvals, dbias, ws, flags, status_flag, st);
   }
   return launch_status();
 }

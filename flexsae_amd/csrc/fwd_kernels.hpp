@@ -114,7 +114,15 @@ __global__ __launch_bounds__(1024) void loss_finalize_kernel(const float *__rest
                                                              float *__restrict__ loss) {
   __shared__ double red[1024];
   double s = 0.0;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) s += static_cast<double>(partial[i]);
+  int64_t i = threadIdx.x;
+  for (; i + 7 * 1024 < n; i += 8 * 1024) {  // eight independent loads in flight
+    float x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) x[u] = partial[i + u * 1024];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += static_cast<double>(x[u]);
+  }
+  for (; i < n; i += 1024) s += static_cast<double>(partial[i]);
   red[threadIdx.x] = s;
   __syncthreads();
   for (int w = 512; w > 0; w >>= 1) {

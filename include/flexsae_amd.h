@@ -53,7 +53,12 @@ enum { FLEXSAE_FLAG_INDEX_RANGE = 1 };
 
 /* flags for the backward entry points */
 enum {
-  FLEXSAE_BWD_OUTPUTS_PREZEROED = 1 /* caller already zero-filled the accumulators */
+  FLEXSAE_BWD_OUTPUTS_PREZEROED = 1, /* caller already zero-filled the accumulators            */
+  /* flexsae_hier_bwd only: */
+  FLEXSAE_BWD_REUSE_PAIR_LIST = 2,   /* the workspace still holds the pair list of a previous   */
+                                     /* call with the same indices and shape: do not rebuild it */
+  FLEXSAE_BWD_SWEEP_ONLY = 4,        /* measurement aid: run only the sweep kernels             */
+  FLEXSAE_BWD_REDUCE_ONLY = 8        /* measurement aid: run only the segment reductions        */
 };
 
 /* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^31; B*K < 2^32. */
