@@ -147,25 +147,30 @@ __global__ __launch_bounds__(256) void csr_sort_short_kernel(const uint32_t *__r
   if (have) map[s0 + rank] = x;  // every lane read its element before any lane writes
 }
 
-// Long groups: in-place bitonic network in which every comparator points the same way
-// (first sub-step of each merge mirrors, the rest are plain strides), so a length that is
-// not a power of two is handled by skipping comparators whose partner lies beyond the end.
-__global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
-                                                            uint32_t *__restrict__ map,
-                                                            const uint32_t *__restrict__ long_count,
-                                                            const uint32_t *__restrict__ long_list) {
-  const uint32_t n_long = *long_count;
-  for (uint32_t w = blockIdx.x; w < n_long; w += gridDim.x) {
-    const uint32_t f = long_list[w];
-    uint32_t *a = map + begin[f];
-    const uint32_t n = begin[f + 1] - begin[f];
-    uint32_t np2 = 1;
-    while (np2 < n) np2 <<= 1;
-    for (uint32_t k = 2; k <= np2; k <<= 1) {
-      // mirrored sub-step: inside each block of k, position i pairs with (k-1-i)
+// Bitonic network in which every comparator points the same way (first sub-step of each merge
+// mirrors, the rest are plain strides), so a length that is not a power of two is handled by
+// skipping comparators whose partner lies beyond the end.  Run by one whole block on a[0..n).
+template <typename Ptr>
+__device__ __forceinline__ void block_bitonic_sort(Ptr a, uint32_t n) {
+  uint32_t np2 = 1;
+  while (np2 < n) np2 <<= 1;
+  for (uint32_t k = 2; k <= np2; k <<= 1) {
+    // mirrored sub-step: inside each block of k, position i pairs with (k-1-i)
+    for (uint32_t t = threadIdx.x; t < np2 / 2; t += blockDim.x) {
+      const uint32_t blk = t / (k / 2), i = t % (k / 2);
+      const uint32_t lo = blk * k + i, hi = blk * k + (k - 1 - i);
+      if (hi < n) {
+        const uint32_t x = a[lo], y = a[hi];
+        if (x > y) {
+          a[lo] = y;
+          a[hi] = x;
+        }
+      }
+    }
+    __syncthreads();
+    for (uint32_t j = k / 4; j > 0; j >>= 1) {
       for (uint32_t t = threadIdx.x; t < np2 / 2; t += blockDim.x) {
-        const uint32_t blk = t / (k / 2), i = t % (k / 2);
-        const uint32_t lo = blk * k + i, hi = blk * k + (k - 1 - i);
+        const uint32_t lo = (t / j) * (2 * j) + (t % j), hi = lo + j;
         if (hi < n) {
           const uint32_t x = a[lo], y = a[hi];
           if (x > y) {
@@ -175,19 +180,31 @@ __global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__re
         }
       }
       __syncthreads();
-      for (uint32_t j = k / 4; j > 0; j >>= 1) {
-        for (uint32_t t = threadIdx.x; t < np2 / 2; t += blockDim.x) {
-          const uint32_t lo = (t / j) * (2 * j) + (t % j), hi = lo + j;
-          if (hi < n) {
-            const uint32_t x = a[lo], y = a[hi];
-            if (x > y) {
-              a[lo] = y;
-              a[hi] = x;
-            }
-          }
-        }
-        __syncthreads();
-      }
+    }
+  }
+}
+
+// Long groups (more than 64 pairs): one block per group, striding over the list.  Groups of up
+// to kSortLdsElems pairs are sorted in LDS, longer ones in place in global memory.
+constexpr uint32_t kSortLdsElems = 8192;
+__global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
+                                                            uint32_t *__restrict__ map,
+                                                            const uint32_t *__restrict__ long_count,
+                                                            const uint32_t *__restrict__ long_list) {
+  __shared__ uint32_t buf[kSortLdsElems];
+  const uint32_t n_long = *long_count;
+  for (uint32_t w = blockIdx.x; w < n_long; w += gridDim.x) {
+    const uint32_t f = long_list[w];
+    uint32_t *a = map + begin[f];
+    const uint32_t n = begin[f + 1] - begin[f];
+    if (n <= kSortLdsElems) {
+      for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) buf[i] = a[i];
+      __syncthreads();
+      block_bitonic_sort(buf, n);
+      for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) a[i] = buf[i];
+      __syncthreads();
+    } else {
+      block_bitonic_sort(a, n);
     }
   }
 }

@@ -16,6 +16,7 @@ namespace {
 constexpr int kBlock = 256;              // threads per block of the wave-per-item kernels
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr size_t kAlign = 256;
+constexpr unsigned kLongBlocks = 1024;    // leading blocks of a reduction launch that serve hot latents
 
 inline bool valid_dtype(int d) { return d == FLEXSAE_F32 || d == FLEXSAE_BF16 || d == FLEXSAE_F16; }
 inline size_t dtype_size(int d) { return d == FLEXSAE_F32 ? 4 : 2; }
@@ -316,14 +317,13 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                          s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F,
                          D);
     if (!do_reduce) continue;
-    hipLaunchKernelGGL((seg_reduce_short_kernel<PT, GT, VEC, 8>),
-                       dim3(static_cast<unsigned>(ceil_div(s->F, kWavesPerBlock))), dim3(kBlock), 0, st,
-                       begin, P, dW, s->F, tps, static_cast<int>(col0), sw, D);
-    hipLaunchKernelGGL((seg_reduce_long_kernel<PT, VEC, 8>), dim3(1024), dim3(kBlock), 0, st, begin,
-                       sc.long_count, sc.long_list, chunk_begin, P, partial, tps, sw);
+    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(s->F, kWavesPerBlock));
+    hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, 8>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock),
+                       0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, s->F,
+                       kLongBlocks, tps, static_cast<int>(col0), sw, D);
     hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
-                       sc.long_count, sc.long_list, chunk_begin, partial, dW, tps,
-                       static_cast<int>(col0), sw, D);
+                       sc.long_count, sc.long_list, chunk_begin, partial, dW, tps, static_cast<int>(col0),
+                       sw, D);
   }
   if (!do_sweep || !do_reduce) return;
   // dbias = column sums of s_final over the rows, in a fixed order
@@ -424,16 +424,13 @@ void launch_topk_slices(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t s
     const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
     const int64_t n_items = s->F * tps;
-    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, VEC, 4>),
-                       dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
-                       begin, map, weight, vals, s->vals_dtype, resid, grad_out, coef, dW, dvals, n_items,
-                       static_cast<int>(col0), s->F, K, D);
-    hipLaunchKernelGGL((topk_bwd_long_kernel<WT, VEC, 4>), dim3(1024), dim3(kBlock), 0, st, begin, map,
-                       long_count, long_list, chunk_begin, weight, vals, s->vals_dtype, resid, grad_out,
-                       coef, dvals, partial, tps, static_cast<int>(col0), sw, K, D);
+    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock));
+    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, VEC, 4>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock), 0,
+                       st, begin, map, long_count, long_list, chunk_begin, weight, vals, s->vals_dtype, resid,
+                       grad_out, coef, dW, dvals, partial, n_items, kLongBlocks, tps, static_cast<int>(col0),
+                       sw, s->F, K, D);
     hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
-                       long_count, long_list, chunk_begin, partial, dW, tps, static_cast<int>(col0), sw,
-                       D);
+                       long_count, long_list, chunk_begin, partial, dW, tps, static_cast<int>(col0), sw, D);
   }
 }
 

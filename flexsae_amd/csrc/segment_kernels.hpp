@@ -1,8 +1,8 @@
 // Latent-major segment reduction: out[f, slice] = sum of the rows [begin[f], begin[f+1]) of
 // P[., slice] (rows of one latent are adjacent), with fp32 accumulation and one write per
 // output element.  Short groups (<= 64 rows) are reduced by one wavefront; long ones are cut
-// into chunks of 64 rows whose fp32 partial sums are combined by a second kernel, so a hot
-// latent is spread over many wavefronts and the summation order stays fixed (deterministic).
+// into chunks of 64 rows whose fp32 partial sums are combined in chunk order, so a hot latent is
+// spread over many wavefronts and the summation order stays fixed (deterministic).
 #pragma once
 
 #include "common.hpp"
@@ -33,26 +33,102 @@ __device__ __forceinline__ void accumulate_rows(const void *__restrict__ X, int6
   }
 }
 
-// One wavefront per latent; it walks the tiles of the slice (64*VEC columns each).  Latents
-// with more than kSegChunk rows are left to the long path; latents without rows get zeros.
+// Decode work item `chunk` of the long-latent work list: which latent, which rows.
+struct LongChunk {
+  uint32_t long_slot;
+  int64_t f;
+  uint32_t s0, s1;  // rows [s0, s1) of the pair list
+};
+__device__ __forceinline__ LongChunk seg_decode_chunk(const uint32_t *__restrict__ begin,
+                                                      const uint32_t *__restrict__ long_list,
+                                                      const uint32_t *__restrict__ chunk_begin,
+                                                      uint32_t n_long, uint32_t chunk) {
+  uint32_t lo = 0, hi = n_long;  // largest i with chunk_begin[i] <= chunk
+  while (hi - lo > 1) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (chunk_begin[mid] <= chunk) lo = mid; else hi = mid;
+  }
+  LongChunk c;
+  c.long_slot = lo;
+  c.f = long_list[lo];
+  c.s0 = begin[c.f] + (chunk - chunk_begin[lo]) * kSegChunk;
+  const uint32_t s_lim = begin[c.f + 1];
+  c.s1 = (s_lim - c.s0) < static_cast<uint32_t>(kSegChunk) ? s_lim : c.s0 + kSegChunk;
+  return c;
+}
+
+// Segment reduction of one slice.
+// Blocks [0, n_long_blocks): long latents.  Every (64-row chunk, tile) is reduced by one
+// wavefront into partial[chunk, slice column] (fp32); the wavefronts stride over the work list,
+// whose length is only known on the device.  seg_reduce_long_finalize_kernel (next launch)
+// combines the partials in chunk order.  These blocks come first so that hot latents start
+// at once and overlap with the bulk of the work.
+// Remaining blocks: one wavefront per latent walks the tiles of the slice (64*VEC columns
+// each); latents without rows get zeros; latents with more than kSegChunk rows are skipped.
 template <typename PT, typename GT, int VEC, int U>
-__global__ __launch_bounds__(256) void seg_reduce_short_kernel(
-    const uint32_t *__restrict__ begin, const void *__restrict__ P, void *__restrict__ out,
-    int64_t F, int tps, int col0, int slice_w, int D) {
+__global__ __launch_bounds__(256) void seg_reduce_kernel(
+    const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
+    const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
+    const void *__restrict__ P, float *__restrict__ partial, void *__restrict__ out, int64_t F,
+    unsigned n_long_blocks, int tps, int col0, int slice_w, int D) {
   const int lane = lane_id();
-  const int64_t f = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
-  if (f >= F) return;  // uniform per wavefront
-  const uint32_t s0 = begin[f];
-  const uint32_t n = begin[f + 1] - s0;
-  if (n > static_cast<uint32_t>(kSegChunk)) return;
-  for (int t = 0; t < tps; ++t) {
+  if (blockIdx.x >= n_long_blocks) {
+    const int64_t f = static_cast<int64_t>(blockIdx.x - n_long_blocks) * (blockDim.x >> 6) + wave_in_block();
+    if (f >= F) return;  // uniform per wavefront
+    const uint32_t s0 = begin[f];
+    const uint32_t n = begin[f + 1] - s0;
+    if (n > static_cast<uint32_t>(kSegChunk)) return;
+    for (int t = 0; t < tps; ++t) {
+      const int pc = t * (kWave * VEC) + lane * VEC;
+      const int d0 = col0 + pc;
+      float acc[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+      accumulate_rows<PT, VEC, U>(P, s0, static_cast<int>(n), slice_w, pc, acc);
+      if (d0 < D) store_vec<GT, VEC>(out, f * D + d0, acc);
+    }
+    return;
+  }
+  const uint32_t n_long = *long_count;
+  if (n_long == 0) return;
+  const int64_t total = static_cast<int64_t>(chunk_begin[n_long]) * tps;
+  const int64_t n_waves = static_cast<int64_t>(n_long_blocks) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total;
+       w += n_waves) {
+    const uint32_t chunk = static_cast<uint32_t>(w / tps);
+    const int t = static_cast<int>(w - static_cast<int64_t>(chunk) * tps);
+    const LongChunk c = seg_decode_chunk(begin, long_list, chunk_begin, n_long, chunk);
     const int pc = t * (kWave * VEC) + lane * VEC;
-    const int d0 = col0 + pc;
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-    accumulate_rows<PT, VEC, U>(P, s0, static_cast<int>(n), slice_w, pc, acc);
-    if (d0 < D) store_vec<GT, VEC>(out, f * D + d0, acc);
+    accumulate_rows<PT, VEC, U>(P, c.s0, static_cast<int>(c.s1 - c.s0), slice_w, pc, acc);
+    store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
+  }
+}
+
+// Long latents, second launch: out[f, slice] = sum of the latent's chunk partials, in chunk order.
+template <typename GT, int VEC, int U>
+__global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
+    const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
+    const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
+    void *__restrict__ out, int tps, int col0, int slice_w, int D) {
+  const int lane = lane_id();
+  const uint32_t n_long = *long_count;
+  const int64_t total = static_cast<int64_t>(n_long) * tps;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total;
+       w += n_waves) {
+    const uint32_t i = static_cast<uint32_t>(w / tps);
+    const int t = static_cast<int>(w - static_cast<int64_t>(i) * tps);
+    const int pc = t * (kWave * VEC) + lane * VEC;
+    const int d0 = col0 + pc;
+    const uint32_t c0 = chunk_begin[i], c1 = chunk_begin[i + 1];
+    float acc[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
+    accumulate_rows<float, VEC, U>(partial, c0, static_cast<int>(c1 - c0), slice_w, pc, acc);
+    if (d0 < D) store_vec<GT, VEC>(out, static_cast<int64_t>(long_list[i]) * D + d0, acc);
   }
 }
 
@@ -103,67 +179,6 @@ __global__ __launch_bounds__(1024) void seg_chunk_table_kernel(const uint32_t *_
     __syncthreads();
   }
   if (tid == 0) chunk_begin[n_long] = carry_s;
-}
-
-// Long latents, step 1: every (chunk, tile) is reduced by one wavefront into
-// partial[chunk, slice] (fp32).  Fixed-size grid; wavefronts stride over the work list, whose
-// length is only known on the device.
-template <typename PT, int VEC, int U>
-__global__ __launch_bounds__(256) void seg_reduce_long_kernel(
-    const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
-    const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
-    const void *__restrict__ P, float *__restrict__ partial, int tps, int slice_w) {
-  const int lane = lane_id();
-  const uint32_t n_long = *long_count;
-  if (n_long == 0) return;
-  const int64_t total = static_cast<int64_t>(chunk_begin[n_long]) * tps;
-  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
-  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total;
-       w += n_waves) {
-    const uint32_t chunk = static_cast<uint32_t>(w / tps);
-    const int t = static_cast<int>(w - static_cast<int64_t>(chunk) * tps);
-    // largest i with chunk_begin[i] <= chunk
-    uint32_t lo = 0, hi = n_long;
-    while (hi - lo > 1) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (chunk_begin[mid] <= chunk) lo = mid; else hi = mid;
-    }
-    const uint32_t f = long_list[lo];
-    const uint32_t s0 = begin[f] + (chunk - chunk_begin[lo]) * kSegChunk;
-    const uint32_t s_end = begin[f + 1];
-    const uint32_t n = (s_end - s0) < static_cast<uint32_t>(kSegChunk) ? (s_end - s0) : kSegChunk;
-    const int pc = t * (kWave * VEC) + lane * VEC;
-    float acc[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-    accumulate_rows<PT, VEC, U>(P, s0, static_cast<int>(n), slice_w, pc, acc);
-    store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
-  }
-}
-
-// Long latents, step 2: out[f, slice] = sum of the latent's chunk partials, in chunk order.
-template <typename GT, int VEC, int U>
-__global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
-    const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
-    const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
-    void *__restrict__ out, int tps, int col0, int slice_w, int D) {
-  const int lane = lane_id();
-  const uint32_t n_long = *long_count;
-  const int64_t total = static_cast<int64_t>(n_long) * tps;
-  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
-  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total;
-       w += n_waves) {
-    const uint32_t i = static_cast<uint32_t>(w / tps);
-    const int t = static_cast<int>(w - static_cast<int64_t>(i) * tps);
-    const int pc = t * (kWave * VEC) + lane * VEC;
-    const int d0 = col0 + pc;
-    const uint32_t c0 = chunk_begin[i], c1 = chunk_begin[i + 1];
-    float acc[VEC];
-#pragma unroll
-    for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
-    accumulate_rows<float, VEC, U>(partial, c0, static_cast<int>(c1 - c0), slice_w, pc, acc);
-    if (d0 < D) store_vec<GT, VEC>(out, static_cast<int64_t>(long_list[i]) * D + d0, acc);
-  }
 }
 
 }  // namespace flexsae

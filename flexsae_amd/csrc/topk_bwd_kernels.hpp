@@ -62,76 +62,36 @@ __device__ __forceinline__ void topk_accumulate_slots(
   }
 }
 
-// One wavefront per (tile of the slice, latent f), tile-major, so that at any moment the waves
-// in flight share one B x tile slice of resid (L2-sized).  tile = 64*VEC columns, lane l owning
-// VEC consecutive columns.  dW[f, tile] is written exactly once, in the gradient's final dtype;
-// latents without pairs get zeros; latents with more than kSegChunk pairs are left to
-// topk_bwd_long_kernel.  scale = grad_out * 2/(B*D).
+// TopK backward of one slice.  scale = grad_out * 2/(B*D).
+// Blocks [0, n_long_blocks): long latents, one wavefront per (64-pair chunk, tile): adds its
+// dvals, leaves its dW contribution in partial[chunk, slice column] (fp32) for
+// seg_reduce_long_finalize_kernel (next launch).  They come first so hot latents start at once.
+// Remaining blocks: one wavefront per (tile of the slice, latent f), tile-major, so that at any
+// moment the waves in flight share one B x tile slice of resid (L2-sized).  tile = 64*VEC
+// columns, lane l owning VEC consecutive columns.  dW[f, tile] is written exactly once, in the
+// gradient's final dtype; latents without pairs get zeros; latents with more than kSegChunk
+// pairs are skipped here.
 template <typename WT, typename GT, int VEC, int U>
 __global__ __launch_bounds__(256) void topk_bwd_kernel(
-    const uint32_t *__restrict__ begin, const uint32_t *__restrict__ map,
-    const void *__restrict__ weight, const void *__restrict__ vals, int vals_dtype,
-    const float *__restrict__ resid, const float *__restrict__ grad_out, float coef,
-    void *__restrict__ dW, float *__restrict__ dvals, int64_t n_items, int col0, int64_t F, int K,
-    int D) {
-  const int lane = lane_id();
-  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
-  if (item >= n_items) return;  // uniform per wavefront
-  const int t = static_cast<int>(item / F);
-  const int64_t f = item - static_cast<int64_t>(t) * F;
-  const uint32_t s_begin = begin[f];
-  const uint32_t s_end = begin[f + 1];
-  if (s_end - s_begin > static_cast<uint32_t>(kSegChunk)) return;
-  const int d0 = col0 + t * (kWave * VEC) + lane * VEC;
-  const bool active = d0 < D;
-  const int dsafe = active ? d0 : 0;
-  const float scale = coef * grad_out[0];
-
-  float w[VEC], acc[VEC];
-  load_vec<WT, VEC>(weight, f * D + dsafe, w);
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    acc[i] = 0.f;
-    if (!active) w[i] = 0.f;
-  }
-  topk_accumulate_slots<VEC, U>(map, vals, vals_dtype, resid, scale, dvals, w, s_begin, s_end, K, D,
-                                dsafe, acc);
-  if (active) store_vec<GT, VEC>(dW, f * D + d0, acc);
-}
-
-// Long latents: every (64-pair chunk, tile of the slice) is handled by one wavefront, which
-// adds its dvals and leaves its dW contribution in partial[chunk, slice column] (fp32) for
-// seg_reduce_long_finalize_kernel.  Fixed-size grid striding over a device-side work list.
-template <typename WT, int VEC, int U>
-__global__ __launch_bounds__(256) void topk_bwd_long_kernel(
     const uint32_t *__restrict__ begin, const uint32_t *__restrict__ map,
     const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
     const uint32_t *__restrict__ chunk_begin, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const float *__restrict__ resid,
-    const float *__restrict__ grad_out, float coef, float *__restrict__ dvals,
-    float *__restrict__ partial, int tps, int col0, int slice_w, int K, int D) {
+    const float *__restrict__ grad_out, float coef, void *__restrict__ dW,
+    float *__restrict__ dvals, float *__restrict__ partial, int64_t n_items, unsigned n_long_blocks,
+    int tps, int col0, int slice_w, int64_t F, int K, int D) {
   const int lane = lane_id();
-  const uint32_t n_long = *long_count;
-  if (n_long == 0) return;
   const float scale = coef * grad_out[0];
-  const int64_t total = static_cast<int64_t>(chunk_begin[n_long]) * tps;
-  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
-  for (int64_t wk = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); wk < total;
-       wk += n_waves) {
-    // tile-major over the work list as well
-    const int t = static_cast<int>(wk / chunk_begin[n_long]);
-    const uint32_t chunk = static_cast<uint32_t>(wk - static_cast<int64_t>(t) * chunk_begin[n_long]);
-    uint32_t lo = 0, hi = n_long;  // largest i with chunk_begin[i] <= chunk
-    while (hi - lo > 1) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (chunk_begin[mid] <= chunk) lo = mid; else hi = mid;
-    }
-    const int64_t f = long_list[lo];
-    const uint32_t s0 = begin[f] + (chunk - chunk_begin[lo]) * kSegChunk;
-    const uint32_t s_lim = begin[f + 1];
-    const uint32_t s1 = (s_lim - s0) < static_cast<uint32_t>(kSegChunk) ? s_lim : s0 + kSegChunk;
-    const int pc = t * (kWave * VEC) + lane * VEC;
-    const int d0 = col0 + pc;
+  if (blockIdx.x >= n_long_blocks) {
+    const int64_t item =
+        static_cast<int64_t>(blockIdx.x - n_long_blocks) * (blockDim.x >> 6) + wave_in_block();
+    if (item >= n_items) return;  // uniform per wavefront
+    const int t = static_cast<int>(item / F);
+    const int64_t f = item - static_cast<int64_t>(t) * F;
+    const uint32_t s_begin = begin[f];
+    const uint32_t s_end = begin[f + 1];
+    if (s_end - s_begin > static_cast<uint32_t>(kSegChunk)) return;
+    const int d0 = col0 + t * (kWave * VEC) + lane * VEC;
     const bool active = d0 < D;
     const int dsafe = active ? d0 : 0;
     float w[VEC], acc[VEC];
@@ -141,7 +101,34 @@ __global__ __launch_bounds__(256) void topk_bwd_long_kernel(
       acc[i] = 0.f;
       if (!active) w[i] = 0.f;
     }
-    topk_accumulate_slots<VEC, U>(map, vals, vals_dtype, resid, scale, dvals, w, s0, s1, K, D, dsafe,
+    topk_accumulate_slots<VEC, U>(map, vals, vals_dtype, resid, scale, dvals, w, s_begin, s_end, K, D,
+                                  dsafe, acc);
+    if (active) store_vec<GT, VEC>(dW, f * D + d0, acc);
+    return;
+  }
+  const uint32_t n_long = *long_count;
+  if (n_long == 0) return;
+  const uint32_t n_chunks = chunk_begin[n_long];
+  const int64_t total = static_cast<int64_t>(n_chunks) * tps;
+  const int64_t n_waves = static_cast<int64_t>(n_long_blocks) * (blockDim.x >> 6);
+  for (int64_t wk = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); wk < total;
+       wk += n_waves) {
+    // tile-major over the work list as well
+    const int t = static_cast<int>(wk / n_chunks);
+    const uint32_t chunk = static_cast<uint32_t>(wk - static_cast<int64_t>(t) * n_chunks);
+    const LongChunk c = seg_decode_chunk(begin, long_list, chunk_begin, n_long, chunk);
+    const int pc = t * (kWave * VEC) + lane * VEC;
+    const int d0 = col0 + pc;
+    const bool active = d0 < D;
+    const int dsafe = active ? d0 : 0;
+    float w[VEC], acc[VEC];
+    load_vec<WT, VEC>(weight, c.f * D + dsafe, w);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      acc[i] = 0.f;
+      if (!active) w[i] = 0.f;
+    }
+    topk_accumulate_slots<VEC, U>(map, vals, vals_dtype, resid, scale, dvals, w, c.s0, c.s1, K, D, dsafe,
                                   acc);
     store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
   }
