@@ -1,6 +1,7 @@
 // C-ABI entry points (include/flexsae_amd.h): argument validation, kernel selection and
 // launches.  No allocation, no synchronisation, no global state.
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
 
 #include "common.hpp"
 #include "fwd_kernels.hpp"
@@ -10,6 +11,20 @@
 #include "topk_bwd_kernels.hpp"
 
 using namespace flexsae;
+
+// gathers in flight per wavefront before the first one is consumed
+#ifndef FLEXSAE_SWEEP_U
+#define FLEXSAE_SWEEP_U 16
+#endif
+#ifndef FLEXSAE_REDUCE_U
+#define FLEXSAE_REDUCE_U 8
+#endif
+#ifndef FLEXSAE_FWD_U
+#define FLEXSAE_FWD_U 8
+#endif
+#ifndef FLEXSAE_TOPK_U
+#define FLEXSAE_TOPK_U 4
+#endif
 
 namespace {
 
@@ -84,7 +99,7 @@ void launch_fwd_t(const flexsae_shape *s, const FwdPlan &p, const int64_t *indic
                   const void *weight, const void *vals, const void *bias, const void *target,
                   float *resid, float *partial, int *status_flag, hipStream_t st) {
   const unsigned grid = static_cast<unsigned>(ceil_div(p.n_items, kWavesPerBlock));
-  hipLaunchKernelGGL((sae_fwd_kernel<WT, VEC, HIER, 8>), dim3(grid), dim3(kBlock), 0, st, indices,
+  hipLaunchKernelGGL((sae_fwd_kernel<WT, VEC, HIER, FLEXSAE_FWD_U>), dim3(grid), dim3(kBlock), 0, st, indices,
                      weight, vals, s->vals_dtype, bias, s->bias_dtype, target, s->target_dtype,
                      resid, partial, status_flag, p.n_items, p.ntiles, static_cast<int>(s->K),
                      s->F, static_cast<int>(s->D));
@@ -311,14 +326,14 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     const int tps = static_cast<int>(cols / pl.tile);
     const int64_t sweep_items = s->B * tps;
     if (do_sweep)
-      hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, 8>),
+      hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, FLEXSAE_SWEEP_U>),
                          dim3(static_cast<unsigned>(ceil_div(sweep_items, kWavesPerBlock))), dim3(kBlock),
                          0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dvals,
                          s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F,
                          D);
     if (!do_reduce) continue;
     const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(s->F, kWavesPerBlock));
-    hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, 8>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock),
+    hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock),
                        0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, s->F,
                        kLongBlocks, tps, static_cast<int>(col0), sw, D);
     hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
@@ -425,7 +440,7 @@ void launch_topk_slices(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t s
     const int tps = static_cast<int>(cols / pl.tile);
     const int64_t n_items = s->F * tps;
     const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock));
-    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, VEC, 4>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock), 0,
+    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, VEC, FLEXSAE_TOPK_U>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock), 0,
                        st, begin, map, long_count, long_list, chunk_begin, weight, vals, s->vals_dtype, resid,
                        grad_out, coef, dW, dvals, partial, n_items, kLongBlocks, tps, static_cast<int>(col0),
                        sw, s->F, K, D);

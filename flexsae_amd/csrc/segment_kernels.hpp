@@ -11,25 +11,26 @@ namespace flexsae {
 
 constexpr int kSegChunk = 64;  // rows per chunk; groups longer than this count as "long"
 
-// acc += sum of rows [r0, r0+n) of X (row stride `ld` elements) over the lane's VEC columns at pc
+// acc += sum of rows [r0, r0+n) of X (row stride `ld` elements) over the lane's VEC columns at pc.
+// Rows are fetched U at a time; a group that reaches past the end re-reads the last row (a cache
+// hit) instead of falling back to one load at a time, so short groups keep all loads in flight.
 template <typename PT, int VEC, int U>
 __device__ __forceinline__ void accumulate_rows(const void *__restrict__ X, int64_t r0, int n,
                                                 int64_t ld, int pc, float (&acc)[VEC]) {
-  int j = 0;
-  for (; j + U <= n; j += U) {
+  for (int j = 0; j < n; j += U) {
     float x[U][VEC];
 #pragma unroll
-    for (int u = 0; u < U; ++u) load_vec<PT, VEC>(X, (r0 + j + u) * ld + pc, x[u]);
+    for (int u = 0; u < U; ++u) {
+      const int jj = (j + u) < n ? (j + u) : (n - 1);
+      load_vec<PT, VEC>(X, (r0 + jj) * ld + pc, x[u]);
+    }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
+      if (j + u < n) {  // uniform
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[i] += x[u][i];
-  }
-  for (; j < n; ++j) {
-    float x[VEC];
-    load_vec<PT, VEC>(X, (r0 + j) * ld + pc, x);
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] += x[i];
+        for (int i = 0; i < VEC; ++i) acc[i] += x[u][i];
+      }
+    }
   }
 }
 

@@ -41,22 +41,18 @@ __device__ __forceinline__ void topk_accumulate_slots(
       if (lane == j) my_dot = dot;
     };
 
-    int j = 0;
-    for (; j + U <= n; j += U) {
+    // U gathers in flight; a group reaching past the end re-reads the last row (a cache hit)
+    for (int j = 0; j < n; j += U) {
       float g[U][VEC];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t brow = bcast_i32(my_b, j + u);
+        const int jj = (j + u) < n ? (j + u) : (n - 1);
+        const int64_t brow = bcast_i32(my_b, jj);
         load_vec<float, VEC>(resid, brow * D + dsafe, g[u]);
       }
 #pragma unroll
-      for (int u = 0; u < U; ++u) step(j + u, g[u]);
-    }
-    for (; j < n; ++j) {
-      float g[VEC];
-      const int64_t brow = bcast_i32(my_b, j);
-      load_vec<float, VEC>(resid, brow * D + dsafe, g);
-      step(j, g);
+      for (int u = 0; u < U; ++u)
+        if (j + u < n) step(j + u, g[u]);  // uniform
     }
     if (slot < s_end) unsafeAtomicAdd(dvals + p, my_dot * scale);
   }
