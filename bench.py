@@ -230,7 +230,12 @@ def main():
     dW = torch.empty(F, D, dtype=dtype, device=dev)
     p_size = 2 if dtype == torch.bfloat16 else 4
     scratch = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
-    slice_cols = max(1, scratch // (B * K * p_size))
+    # same decision as the API: the fused training step runs when the stage budget holds every
+    # per-pair contribution at once (one slice as wide as D); otherwise forward + sliced backward
+    fused = (os.environ.get("FLEXSAE_FUSED_TRAINING", "1") not in ("", "0") and scratch > 0
+             and flex.ops._stage_fits(idx, W) and flex.ops._train_supported(W, K)
+             and bool(lib.flexsae_hier_fwd_bwd_supported(ctypes.byref(sh))))
+    slice_cols = D if fused else max(1, scratch // (B * K * p_size))
     bws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
     bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
     tile = 64 * (4 if D % 4 == 0 else 2 if D % 2 == 0 else 1)
@@ -249,7 +254,20 @@ def main():
 
     PRE, REUSE, SWEEP, REDUCE = 1, 2, 4, 8
     fwd_k_ms = time_kernel_events(torch, lambda: None, fwd_launch, args.steps, args.warmup)
-    if scratch > 0:
+    step_entry_ms = None
+    if fused:
+        # the API step above went through the fused training-step entry point: time it and its phases
+        def train_launch(flags=0):
+            _lib.check(lib.flexsae_hier_fwd_bwd(ctypes.byref(sh), p(idx), p(W), p(v), p(b), p(t), p(loss), p(dW),
+                                                DT[dtype], p(dvals), p(dbias), p(bws), bws_bytes, flags, None,
+                                                st()), "flexsae_hier_fwd_bwd")
+
+        step_entry_ms = time_kernel_events(torch, lambda: None, train_launch, args.steps, args.warmup)
+        sweep_ms = time_kernel_events(torch, lambda: None, lambda: train_launch(PRE | REUSE | SWEEP), args.steps, 1)
+        reduce_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(PRE | REUSE | REDUCE), args.steps, 1)
+        bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
+        sweep_name = "hier_train_kernel"
+    elif scratch > 0:
         bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
         # the pair list is in the workspace now: time the two phases alone (n_slices launches each)
         sweep_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(PRE | REUSE | SWEEP), args.steps, 1)
@@ -278,15 +296,16 @@ def main():
 
     # algorithmic bytes of ONE sweep launch: its share of the gathered rows, indices/vals/slots,
     # and the residual slice (the staged contributions are traffic, not algorithmic bytes)
+    # (the training-step kernel reads bias/target instead of the residual: same order of bytes)
     sweep_launch_bytes = (B * K * D * es + B * K * (8 + es + 4) * n_slices + B * D * 4) / n_slices
     sweep_launch_ms = sweep_ms / n_slices
     traffic = None
     traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file) and not args.shape:
         with open(traffic_file) as fh:
-            rec = json.load(fh).get(f"{args.workload}:{scratch >> 20}")
+            rec = json.load(fh).get(f"{args.workload}:{'fused' if fused else scratch >> 20}")
         if rec:
-            traffic = rec["hier_sweep_kernel_bytes_per_launch"]
+            traffic = rec.get(f"{sweep_name}_bytes_per_launch")
     roofline = {
         "bound": "hbm",
         "kernel": sweep_name,
@@ -315,7 +334,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
                                f"indices {dist}", "B": B, "K": K, "F": F, "D": D,
-                   "hier_scratch_mb": scratch >> 20},
+                   "hier_scratch_mb": scratch >> 20, "fused_training_step": bool(fused),
+                   "hier_stage_mb": int(os.environ.get("FLEXSAE_HIER_STAGE_MB", "4096"))},
         "roofline": roofline,
         "step_hbm": {"algorithmic_bytes": abytes["hier_step"],
                      "achieved_GBps": round(gbps(abytes["hier_step"], hier_ms), 1),
@@ -328,6 +348,8 @@ def main():
             "flexsae_hier_bwd (pair list + sweep + reduce)": {
                 "ms": round(bwd_k_ms, 4), "algorithmic_bytes": abytes["hier_bwd_kernel"],
                 "GBps": round(gbps(abytes["hier_bwd_kernel"], bwd_k_ms), 1)},
+            "flexsae_hier_fwd_bwd (fused training step: pair list + train kernel + reduce)": (
+                {"ms": round(step_entry_ms, 4)} if step_entry_ms is not None else None),
             "%s x%d" % (sweep_name, n_slices): {"ms": round(sweep_ms, 4)},
             "segment reduction x%d" % n_slices: {"ms": round(reduce_ms, 4)},
         },

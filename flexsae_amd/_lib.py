@@ -25,6 +25,10 @@ F32, BF16, F16 = 0, 1, 2
 
 FLAG_INDEX_RANGE = 1
 BWD_OUTPUTS_PREZEROED = 1
+BWD_REUSE_PAIR_LIST = 2
+BWD_SWEEP_ONLY = 4
+BWD_REDUCE_ONLY = 8
+BWD_SCALE_BY_GRAD_OUT = 16
 
 
 class Shape(ctypes.Structure):
@@ -56,6 +60,9 @@ SIGNATURES = {
     "flexsae_topk_fwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _p, _p]),
     "flexsae_hier_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_hier_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p, _p]),
+    "flexsae_hier_fwd_bwd_supported": (_int, [_shape_p]),
+    "flexsae_hier_fwd_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p, _p]),
+    "flexsae_scale": (_int, [_p, _p, _int, _i64, _p, _p]),
     "flexsae_hier_bwd_atomic": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p]),
     "flexsae_csr_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "flexsae_csr_build": (_int, [_p, _i64, _i64, _i64, _p, _p, _p, _sz, _p, _p]),

@@ -7,6 +7,7 @@
 #include "fwd_kernels.hpp"
 #include "csr_kernels.hpp"
 #include "hier_bwd_kernels.hpp"
+#include "hier_train_kernel.hpp"
 #include "segment_kernels.hpp"
 #include "topk_bwd_kernels.hpp"
 
@@ -258,7 +259,8 @@ struct HierBwdPlan {
   size_t n_pairs;          // B * K
   size_t n_rows;           // B
   size_t n_partial_rows;   // upper bound on the number of 64-pair chunks of long latents
-  size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_sfinal, off_colsum, off_partial;  // per-slice buffers follow
+  size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_sfinal, off_colsum, off_loss, off_partial;  // per-slice buffers follow
+  size_t n_loss_partials;  // training-step kernel: one per (128-column tile, row)
   size_t fixed_bytes;      // everything that does not depend on the slice width
 };
 
@@ -286,9 +288,58 @@ HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
   off += round_up(p.n_rows * static_cast<size_t>(p.d_pad) * 4, kAlign);
   p.off_colsum = off;  // partial column sums, [ceil(B/64), D] fp32
   off += round_up(static_cast<size_t>(ceil_div(s->B, kColsumRows)) * static_cast<size_t>(s->D) * 4, kAlign);
+  p.off_loss = off;
+  p.n_loss_partials = p.n_rows * static_cast<size_t>(p.d_pad / 128 + 1);
+  off += round_up(p.n_loss_partials * 4, kAlign);
   p.off_partial = off;
   p.fixed_bytes = off;
   return p;
+}
+
+// Forward-only inputs of the training-step variant of the slice loop (null = plain backward).
+struct TrainArgs {
+  const void *bias;
+  const void *target;
+};
+
+// largest K the training-step kernel holds in registers, per weight dtype
+inline int train_kmax(int weight_dtype) { return weight_dtype == FLEXSAE_F32 ? 64 : 128; }
+inline bool train_supported(const flexsae_shape *s) {
+  return s->D % 4 == 0 && s->K <= train_kmax(s->weight_dtype);
+}
+
+template <typename WT, typename PT, int KMAX>
+void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
+                         const void *weight, const void *vals, float coef, const uint32_t *slot, void *P,
+                         float *dvals, float *s_final, int d_pad, float *loss_partial, int *status_flag,
+                         int64_t cols, int col0, int slice_w, hipStream_t st) {
+  const int64_t n_items = s->B * (cols / 128);
+  hipLaunchKernelGGL((hier_train_kernel<WT, PT, KMAX>),
+                     dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
+                     indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
+                     coef, slot, P, dvals, s_final, d_pad, loss_partial, status_flag, n_items, s->B, col0,
+                     slice_w, static_cast<int>(s->K), s->F, static_cast<int>(s->D));
+}
+
+template <typename WT, typename PT>
+void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
+                           const void *weight, const void *vals, float coef, const uint32_t *slot, void *P,
+                           float *dvals, float *s_final, int d_pad, float *loss_partial,
+                           int *status_flag, int64_t cols, int col0, int slice_w, hipStream_t st) {
+#define FLEXSAE_TRAIN(KM)                                                                              \
+  launch_train_kernel<WT, PT, KM>(s, ta, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,  \
+                                  loss_partial, status_flag, cols, col0, slice_w, st)
+  // (the fp32 16-step instantiation allocates registers badly; 32 covers it)
+  if (s->K <= 16 && sizeof(typename Traits<WT>::store_t) == 2) {
+    FLEXSAE_TRAIN(16);
+  } else if (s->K <= 32) {
+    FLEXSAE_TRAIN(32);
+  } else if (s->K <= 64) {
+    FLEXSAE_TRAIN(64);
+  } else {
+    if constexpr (sizeof(typename Traits<WT>::store_t) == 2) FLEXSAE_TRAIN(128);
+  }
+#undef FLEXSAE_TRAIN
 }
 
 // per-slice buffers after the fixed part: chunk partials[n_partial_rows, w] | P[B*K, w]
@@ -306,9 +357,10 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                         const int64_t *indices, const void *weight, const void *vals,
                         const float *resid, const float *grad_out, float coef, void *dW,
                         float *dvals, float *dbias, uint8_t *ws, int flags, int *status_flag,
-                        hipStream_t st) {
+                        hipStream_t st, const TrainArgs *train = nullptr) {
   const bool do_sweep = !(flags & FLEXSAE_BWD_REDUCE_ONLY);
   const bool do_reduce = !(flags & FLEXSAE_BWD_SWEEP_ONLY);
+  const float *dw_scale = (flags & FLEXSAE_BWD_SCALE_BY_GRAD_OUT) ? grad_out : nullptr;
   const uint32_t *begin = reinterpret_cast<const uint32_t *>(ws + pl.off_begin);
   const uint32_t *slot = reinterpret_cast<const uint32_t *>(ws + pl.off_slot);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
@@ -325,7 +377,11 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
     const int64_t sweep_items = s->B * tps;
-    if (do_sweep)
+    if (train && do_sweep) {
+      launch_train_kernel_k<WT, PT>(s, *train, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,
+                                    reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
+                                    static_cast<int>(col0), sw, st);
+    } else if (do_sweep)
       hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, FLEXSAE_SWEEP_U>),
                          dim3(static_cast<unsigned>(ceil_div(sweep_items, kWavesPerBlock))), dim3(kBlock),
                          0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dvals,
@@ -334,13 +390,14 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     if (!do_reduce) continue;
     const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(s->F, kWavesPerBlock));
     hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock),
-                       0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, s->F,
+                       0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, s->F,
                        kLongBlocks, tps, static_cast<int>(col0), sw, D);
     hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
-                       sc.long_count, sc.long_list, chunk_begin, partial, dW, tps, static_cast<int>(col0),
-                       sw, D);
+                       sc.long_count, sc.long_list, chunk_begin, partial, dW, dw_scale, tps,
+                       static_cast<int>(col0), sw, D);
   }
-  if (!do_sweep || !do_reduce) return;
+  if (!do_sweep) return;
+  if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
   // dbias = column sums of s_final over the rows, in a fixed order
   hipLaunchKernelGGL(colsum_partial_kernel,
                      dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
@@ -354,19 +411,19 @@ void launch_hier_slices_g(const flexsae_shape *s, const HierBwdPlan &pl, int64_t
                           const int64_t *indices, const void *weight, const void *vals,
                           const float *resid, const float *grad_out, float coef, void *dW,
                           int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int flags,
-                          int *status_flag, hipStream_t st) {
+                          int *status_flag, hipStream_t st, const TrainArgs *train) {
   switch (dW_dtype) {
     case FLEXSAE_F32:
       launch_hier_slices<WT, PT, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                             coef, dW, dvals, dbias, ws, flags, status_flag, st);
+                                             coef, dW, dvals, dbias, ws, flags, status_flag, st, train);
       break;
     case FLEXSAE_BF16:
       launch_hier_slices<WT, PT, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dvals, dbias, ws, flags, status_flag, st);
+                                              coef, dW, dvals, dbias, ws, flags, status_flag, st, train);
       break;
     default:
       launch_hier_slices<WT, PT, f16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                             coef, dW, dvals, dbias, ws, flags, status_flag, st);
+                                             coef, dW, dvals, dbias, ws, flags, status_flag, st, train);
   }
 }
 
@@ -375,19 +432,19 @@ void launch_hier_slices_w(const flexsae_shape *s, const HierBwdPlan &pl, int64_t
                           const int64_t *indices, const void *weight, const void *vals,
                           const float *resid, const float *grad_out, float coef, void *dW,
                           int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int flags,
-                          int *status_flag, hipStream_t st) {
+                          int *status_flag, hipStream_t st, const TrainArgs *train = nullptr) {
   switch (s->weight_dtype) {
     case FLEXSAE_F32:
       launch_hier_slices_g<float, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st);
+                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train);
       break;
     case FLEXSAE_BF16:
       launch_hier_slices_g<bf16_t, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                                coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st);
+                                                coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train);
       break;
     default:
       launch_hier_slices_g<f16_t, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st);
+                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train);
   }
 }
 
@@ -445,7 +502,8 @@ void launch_topk_slices(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t s
                        grad_out, coef, dW, dvals, partial, n_items, kLongBlocks, tps, static_cast<int>(col0),
                        sw, s->F, K, D);
     hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
-                       long_count, long_list, chunk_begin, partial, dW, tps, static_cast<int>(col0), sw, D);
+                       long_count, long_list, chunk_begin, partial, dW, static_cast<const float *>(nullptr), tps,
+                       static_cast<int>(col0), sw, D);
   }
 }
 
@@ -586,24 +644,32 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
                      size_t workspace_bytes, int flags, int *status_flag, void *stream) {
   int rc = check_shape(s);
   if (rc != FLEXSAE_OK) return rc;
-  if (!indices || !weight || !vals || !resid || !grad_out || !dW || !dvals || !dbias ||
-      !valid_dtype(dW_dtype))
-    return FLEXSAE_ERR_INVALID_ARGUMENT;
+  if (!grad_out || !dW || !valid_dtype(dW_dtype)) return FLEXSAE_ERR_INVALID_ARGUMENT;
   const HierBwdPlan pl = plan_hier_bwd(s);
-  if (!aligned(indices, 8) || !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
-      !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.vec * 4) ||
-      !aligned(grad_out, 4) || !aligned(dW, pl.vec * dtype_size(dW_dtype)) || !aligned(dvals, 16) ||
-      !aligned(dbias, 16))
-    return FLEXSAE_ERR_ALIGNMENT;
   if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, pl.tile))
     return FLEXSAE_ERR_WORKSPACE;
   // widest slice (whole tiles) the workspace can hold
   int64_t slice_w = pl.tile;
   while (slice_w + pl.tile <= pl.d_pad && hier_bwd_bytes(pl, slice_w + pl.tile) <= workspace_bytes)
     slice_w += pl.tile;
+  // REDUCE_ONLY on a kept pair list: with a single-slice workspace this is the deferred reduction
+  // of staged contributions, which only reads the workspace and writes dW; on a sliced workspace
+  // it is the reduction phase of every slice (profiling), which still needs the other arguments
+  const bool reduce_only = (flags & FLEXSAE_BWD_REDUCE_ONLY) && (flags & FLEXSAE_BWD_REUSE_PAIR_LIST) &&
+                           slice_w >= pl.d_pad;
+  if (!reduce_only && (!indices || !weight || !vals || !resid || !dvals || !dbias))
+    return (flags & FLEXSAE_BWD_SCALE_BY_GRAD_OUT) ? FLEXSAE_ERR_WORKSPACE : FLEXSAE_ERR_INVALID_ARGUMENT;
+  if ((flags & FLEXSAE_BWD_SCALE_BY_GRAD_OUT) && !reduce_only)
+    return slice_w < pl.d_pad ? FLEXSAE_ERR_WORKSPACE : FLEXSAE_ERR_INVALID_ARGUMENT;
+  if (!aligned(grad_out, 4) || !aligned(dW, pl.vec * dtype_size(dW_dtype))) return FLEXSAE_ERR_ALIGNMENT;
+  if (!reduce_only &&
+      (!aligned(indices, 8) || !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
+       !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.vec * 4) || !aligned(dvals, 16) ||
+       !aligned(dbias, 16)))
+    return FLEXSAE_ERR_ALIGNMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint8_t *ws = static_cast<uint8_t *>(workspace);
-  if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) zero_f32(dvals, s->B * s->K, st);
+  if (!(flags & (FLEXSAE_BWD_OUTPUTS_PREZEROED | FLEXSAE_BWD_REDUCE_ONLY))) zero_f32(dvals, s->B * s->K, st);
   uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
@@ -625,6 +691,81 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   } else {
     launch_hier_slices_w<1>(s, pl, slice_w, indices, weight, vals, resid, grad_out, coef, dW, dW_dtype,
                             dvals, dbias, ws, flags, status_flag, st);
+  }
+  return launch_status();
+}
+
+int flexsae_hier_fwd_bwd_supported(const flexsae_shape *s) {
+  return check_shape(s) == FLEXSAE_OK && train_supported(s) ? 1 : 0;
+}
+
+int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const void *weight,
+                         const void *vals, const void *bias, const void *target, float *loss,
+                         void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
+                         size_t workspace_bytes, int flags, int *status_flag, void *stream) {
+  int rc = check_shape(s);
+  if (rc != FLEXSAE_OK) return rc;
+  const bool defer_reduce = (flags & FLEXSAE_BWD_SWEEP_ONLY) != 0;
+  if (!indices || !weight || !vals || !bias || !target || !loss || !dvals || !dbias ||
+      (!defer_reduce && (!dW || !valid_dtype(dW_dtype))))
+    return FLEXSAE_ERR_INVALID_ARGUMENT;
+  if (!train_supported(s)) return FLEXSAE_ERR_UNSUPPORTED;
+  const HierBwdPlan pl = plan_hier_bwd(s);  // D % 4 == 0 here, so tiles are 256 columns
+  if (!aligned(indices, 8) || !aligned(weight, 4 * dtype_size(s->weight_dtype)) ||
+      !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(bias, 2 * dtype_size(s->bias_dtype)) ||
+      !aligned(target, 2 * dtype_size(s->target_dtype)) || !aligned(loss, 4) ||
+      (!defer_reduce && !aligned(dW, 4 * dtype_size(dW_dtype))) || !aligned(dvals, 16) ||
+      !aligned(dbias, 16))
+    return FLEXSAE_ERR_ALIGNMENT;
+  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, pl.tile))
+    return FLEXSAE_ERR_WORKSPACE;
+  int64_t slice_w = pl.tile;
+  while (slice_w + pl.tile <= pl.d_pad && hier_bwd_bytes(pl, slice_w + pl.tile) <= workspace_bytes)
+    slice_w += pl.tile;
+  if (defer_reduce && slice_w < pl.d_pad) return FLEXSAE_ERR_WORKSPACE;  // contributions must all fit
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
+  if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) zero_f32(dvals, s->B * s->K, st);
+  uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
+  uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
+  if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
+    csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
+    hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
+                       s->B * s->K, reinterpret_cast<uint32_t *>(ws + pl.off_slot));
+    hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
+                       sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+  }
+  const double count = static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D);
+  const float coef = static_cast<float>(2.0 / count);
+  const TrainArgs ta = {bias, target};
+  launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, nullptr, coef, dW, dW_dtype, dvals,
+                          dbias, ws, flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY), status_flag,
+                          st, &ta);
+  rc = launch_status();
+  if (rc != FLEXSAE_OK) return rc;
+  hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(1024), 0, st,
+                     reinterpret_cast<const float *>(ws + pl.off_loss), s->B * (pl.d_pad / 128), 1.0 / count,
+                     loss);
+  return launch_status();
+}
+
+int flexsae_scale(void *dst, const void *src, int dtype, int64_t n, const float *scale, void *stream) {
+  if (!dst || !src || !scale || n < 0 || !valid_dtype(dtype)) return FLEXSAE_ERR_INVALID_ARGUMENT;
+  if (n == 0) return FLEXSAE_OK;
+  if (!aligned(src, 4 * dtype_size(dtype)) || !aligned(dst, 4 * dtype_size(dtype)) || !aligned(scale, 4))
+    return FLEXSAE_ERR_ALIGNMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid(grid_for(ceil_div(n, 4), 256, 1 << 16));
+  switch (dtype) {
+    case FLEXSAE_F32:
+      hipLaunchKernelGGL(scale_kernel<float>, grid, dim3(256), 0, st, dst, src, n, scale);
+      break;
+    case FLEXSAE_BF16:
+      hipLaunchKernelGGL(scale_kernel<bf16_t>, grid, dim3(256), 0, st, dst, src, n, scale);
+      break;
+    default:
+      hipLaunchKernelGGL(scale_kernel<f16_t>, grid, dim3(256), 0, st, dst, src, n, scale);
   }
   return launch_status();
 }

@@ -1,0 +1,242 @@
+// HierarchicalTopK, forward and reverse walk in one kernel ("training step" kernel).
+#pragma once
+
+#include "common.hpp"
+
+namespace flexsae {
+
+// A gathered piece of a weight row (two consecutive columns) kept in raw form.
+template <typename WT>
+struct RowPiece2;
+template <>
+struct RowPiece2<float> {
+  using raw_t = vec_t<float, 2>;
+  static __device__ __forceinline__ void unpack(const raw_t &r, float (&w)[2]) {
+    w[0] = r[0];
+    w[1] = r[1];
+  }
+  // hides the value from common-subexpression elimination (see the kernel)
+  static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
+};
+template <>
+struct RowPiece2<bf16_t> {
+  using raw_t = uint32_t;
+  static __device__ __forceinline__ void unpack(const raw_t &r, float (&w)[2]) {
+    w[0] = __uint_as_float(r << 16);
+    w[1] = __uint_as_float(r & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
+};
+template <>
+struct RowPiece2<f16_t> {
+  using raw_t = uint32_t;
+  static __device__ __forceinline__ void unpack(const raw_t &r, float (&w)[2]) {
+    w[0] = f16_bits_to_f32(static_cast<uint16_t>(r & 0xffffu));
+    w[1] = f16_bits_to_f32(static_cast<uint16_t>(r >> 16));
+  }
+  static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
+};
+
+// Sum over the 64 lanes of eight values per lane at once: returns, in lane L, the wave-wide
+// total of d[L & 7].  Three exchange stages inside each group of 8 lanes halve the number of
+// live values while doubling the lanes summed (partner L^7, then L^2, then L^1: together they
+// generate the whole group), then three stages add the eight groups (L^8 by a row rotation,
+// L^16 and L^32 by lane permutes).  About 3.5 VALU operations per value instead of 12.
+__device__ __forceinline__ float wave_sum8_transposed(const float (&d)[8]) {
+  const int lane = lane_id();
+  const bool b2 = (lane & 4) != 0, b1 = (lane & 2) != 0, b0 = (lane & 1) != 0;
+  float r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float keep = b2 ? d[i + 4] : d[i];
+    const float give = b2 ? d[i] : d[i + 4];
+    r[i] = keep + dpp_move<0x141>(give);  // row_half_mirror: lane ^ 7
+  }
+  float q[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float keep = b1 ? r[i + 2] : r[i];
+    const float give = b1 ? r[i] : r[i + 2];
+    q[i] = keep + dpp_move<0x4E>(give);  // quad_perm [2,3,0,1]: lane ^ 2
+  }
+  const float keep = b0 ? q[1] : q[0];
+  const float give = b0 ? q[0] : q[1];
+  float z = keep + dpp_move<0xB1>(give);  // quad_perm [1,0,3,2]: lane ^ 1
+  z += dpp_move<0x128>(z);                // row_ror:8 within the 16-lane row: lane ^ 8
+  z += __shfl_xor(z, 16, kWave);
+  z += __shfl_xor(z, 32, kWave);
+  return z;
+}
+
+// One wavefront per (tile of the slice, row b), tile-major; a tile is 128 columns and lane l owns
+// columns 2l, 2l+1.  The wavefront issues the gathers of all K row pieces at once (the memory
+// pipeline keeps up to 63 of them in flight per wavefront, so a few wavefronts per SIMD cover the
+// latency), keeps the pieces in registers -- one register per row for 16-bit weights -- and walks
+// them twice:
+//   forward  k = 0..K-1 : e += v_k w_k ; loss += e^2             (e starts as bias - target)
+//   reverse  k = K-1..0 : S += c e ; P[slot_k] = v_k S ; dvals_k = <w_k, S> ; e -= v_k w_k
+// i.e. sae_fwd_kernel and hier_sweep_kernel sharing one gather.  The gradient quantities are
+// those of a unit upstream gradient (c = 2/(B*K*D)); the caller scales them afterwards.
+// KMAX bounds K at compile time so that the row pieces can live in registers; steps k >= K
+// are skipped by uniform branches.  Every block of eight steps reduces its eight dvals dot
+// products with one transposed wave reduction.
+template <typename WT, typename PT, int KMAX>
+__global__ __launch_bounds__(256) void hier_train_kernel(
+    const int64_t *__restrict__ indices, const void *__restrict__ weight,
+    const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
+    const void *__restrict__ target, int target_dtype, float coef,
+    const uint32_t *__restrict__ slot, void *__restrict__ P, float *__restrict__ dvals,
+    float *__restrict__ s_final, int s_final_ld, float *__restrict__ loss_partial,
+    int *status_flag, int64_t n_items, int64_t B, int col0, int slice_w, int K, int64_t F, int D) {
+  using Piece = RowPiece2<WT>;
+  using raw_t = typename Piece::raw_t;
+  using S_t = typename Traits<WT>::store_t;
+  constexpr int VEC = 2;
+  constexpr int KC = (KMAX + kWave - 1) / kWave;  // 64-step chunks held per lane
+  static_assert(KMAX % 8 == 0, "KMAX must be a multiple of 8");
+  const int lane = lane_id();
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+  if (item >= n_items) return;  // uniform per wavefront
+  const int t = static_cast<int>(item / B);
+  const int64_t b = item - static_cast<int64_t>(t) * B;
+  const int pc = t * (kWave * VEC) + lane * VEC;  // column inside the slice
+  const int d0 = col0 + pc;
+  const bool active = d0 < D;
+  const int dsafe = active ? d0 : 0;
+  const int64_t pair0 = b * K;
+
+  int my_row[KC], my_slot[KC];
+  float my_val[KC], my_dval[KC];
+#pragma unroll
+  for (int c = 0; c < KC; ++c) {
+    const int kk = c * kWave + lane;
+    int64_t idx = 0;
+    my_val[c] = 0.f;
+    my_slot[c] = 0;
+    my_dval[c] = 0.f;
+    if (kk < K) {
+      idx = indices[pair0 + kk];
+      my_val[c] = load_scalar(vals, vals_dtype, pair0 + kk);
+      my_slot[c] = static_cast<int>(slot[pair0 + kk]);
+    }
+    if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(F)) {
+      if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
+      idx = 0;
+      my_val[c] = 0.f;
+    }
+    my_row[c] = static_cast<int>(idx);
+  }
+
+  // all gathers at once
+  raw_t raw[KMAX];
+  const S_t *__restrict__ W = static_cast<const S_t *>(weight);
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    if (k < K) {  // uniform
+      const int64_t row = bcast_i32(my_row[k / kWave], k % kWave);
+      raw[k] = *reinterpret_cast<const raw_t *>(W + row * D + dsafe);
+    }
+  }
+
+  float e[VEC], tt[VEC], acc[VEC];
+  load_vec_dyn<WT, VEC>(bias, bias_dtype, dsafe, e);
+  load_vec_dyn<WT, VEC>(target, target_dtype, b * D + dsafe, tt);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    e[i] -= tt[i];
+    acc[i] = 0.f;
+  }
+
+  // forward walk
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    if (k < K) {  // uniform
+      const float v = bcast_f32(my_val[k / kWave], k % kWave);
+      float w[VEC];
+      Piece::unpack(raw[k], w);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        e[i] = fmaf(w[i], v, e[i]);
+        acc[i] = fmaf(e[i], e[i], acc[i]);
+      }
+    }
+  }
+  float lsum = active ? (acc[0] + acc[1]) : 0.f;
+  lsum = wave_sum_lane63(lsum);
+  // one partial per (global tile, row); the finalize kernel adds them in a fixed order
+  if (lane == kWave - 1) loss_partial[(static_cast<int64_t>(col0 / (kWave * VEC)) + t) * B + b] = lsum;
+
+  // reverse walk, eight steps per dvals reduction
+  float S[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) S[i] = 0.f;
+#pragma unroll
+  for (int k8 = KMAX - 8; k8 >= 0; k8 -= 8) {
+    if (k8 < K) {  // uniform
+      float dots[8];
+#pragma unroll
+      for (int u = 7; u >= 0; --u) {
+        const int k = k8 + u;
+        dots[u] = 0.f;
+        if (k < K) {  // uniform
+          const float v = bcast_f32(my_val[k / kWave], k % kWave);
+          const int64_t prow = static_cast<uint32_t>(bcast_i32(my_slot[k / kWave], k % kWave));
+          // Without this the compiler reuses the unpacked values of the forward walk, which
+          // doubles the registers held across the two walks; re-unpacking costs one op per value.
+          raw_t rk = raw[k];
+          Piece::launder(rk);
+          float w[VEC], contrib[VEC];
+          Piece::unpack(rk, w);
+          float dot = 0.f;
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) {
+            S[i] = fmaf(coef, e[i], S[i]);
+            contrib[i] = S[i] * v;
+            dot = fmaf(w[i], S[i], dot);
+            e[i] = fmaf(-w[i], v, e[i]);
+          }
+          if (active) store_vec<PT, VEC>(P, prow * slice_w + pc, contrib);
+          dots[u] = active ? dot : 0.f;
+        }
+      }
+      const float tot = wave_sum8_transposed(dots);  // lane L: total of step k8 + (L & 7)
+      if ((lane >> 3) == ((k8 % kWave) >> 3)) my_dval[k8 / kWave] = tot;
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < KC; ++c) {
+    const int kk = c * kWave + lane;
+    if (kk < K) unsafeAtomicAdd(dvals + pair0 + kk, my_dval[c]);
+  }
+  if (!active) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) S[i] = 0.f;
+  }
+  store_vec<float, VEC>(s_final, b * s_final_ld + col0 + pc, S);
+}
+
+// dst[i] = src[i] * scale[0] (dtype in, same dtype out); used to apply the upstream gradient to
+// the unit-gradient results of the training-step kernel.
+template <typename T>
+__global__ void scale_kernel(void *__restrict__ dst, const void *__restrict__ src, int64_t n,
+                             const float *__restrict__ scale) {
+  const float g = scale[0];
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t n4 = n >> 2;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    float x[4];
+    load_vec<T, 4>(src, i * 4, x);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) x[k] *= g;
+    store_vec<T, 4>(dst, i * 4, x);
+  }
+  for (int64_t i = (n4 << 2) + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    float x[1];
+    load_vec<T, 1>(src, i, x);
+    x[0] *= g;
+    store_vec<T, 1>(dst, i, x);
+  }
+}
+
+}  // namespace flexsae

@@ -70,8 +70,9 @@ template <typename PT, typename GT, int VEC, int U>
 __global__ __launch_bounds__(256) void seg_reduce_kernel(
     const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
     const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
-    const void *__restrict__ P, float *__restrict__ partial, void *__restrict__ out, int64_t F,
-    unsigned n_long_blocks, int tps, int col0, int slice_w, int D) {
+    const void *__restrict__ P, float *__restrict__ partial, void *__restrict__ out,
+    const float *__restrict__ scale, int64_t F, unsigned n_long_blocks, int tps, int col0,
+    int slice_w, int D) {
   const int lane = lane_id();
   if (blockIdx.x >= n_long_blocks) {
     const int64_t f = static_cast<int64_t>(blockIdx.x - n_long_blocks) * (blockDim.x >> 6) + wave_in_block();
@@ -86,6 +87,11 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
 #pragma unroll
       for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
       accumulate_rows<PT, VEC, U>(P, s0, static_cast<int>(n), slice_w, pc, acc);
+      if (scale) {  // the rows were produced for a unit upstream gradient
+        const float g = scale[0];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] *= g;
+      }
       if (d0 < D) store_vec<GT, VEC>(out, f * D + d0, acc);
     }
     return;
@@ -113,7 +119,7 @@ template <typename GT, int VEC, int U>
 __global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
     const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
     const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
-    void *__restrict__ out, int tps, int col0, int slice_w, int D) {
+    void *__restrict__ out, const float *__restrict__ scale, int tps, int col0, int slice_w, int D) {
   const int lane = lane_id();
   const uint32_t n_long = *long_count;
   const int64_t total = static_cast<int64_t>(n_long) * tps;
@@ -129,6 +135,11 @@ __global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
 #pragma unroll
     for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
     accumulate_rows<float, VEC, U>(partial, c0, static_cast<int>(c1 - c0), slice_w, pc, acc);
+    if (scale) {
+      const float g = scale[0];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) acc[k] *= g;
+    }
     if (d0 < D) store_vec<GT, VEC>(out, static_cast<int64_t>(long_list[i]) * D + d0, acc);
   }
 }

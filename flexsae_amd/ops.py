@@ -164,9 +164,24 @@ _hier_scratch_bytes = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 2
 
 def set_hier_scratch_bytes(nbytes: int) -> None:
     """Upper bound on the scratch of the hierarchical backward (bytes).  0 = use the atomic
-    scatter fallback, which needs no scratch but an fp32 [F,D] accumulator."""
+    scatter fallback, which needs no scratch but an fp32 [F,D] accumulator.  The default (256 MiB)
+    is the size at which one slice of contributions stays in the memory-side cache between the
+    sweep that writes it and the reduction that reads it; wider slices run slower, not faster."""
     global _hier_scratch_bytes
     _hier_scratch_bytes = int(nbytes)
+
+
+# Memory the fused training step may hold between forward and backward: all B*K*D per-pair
+# contributions (2 bytes each for bf16 weights, else 4) plus the pair list.
+_hier_stage_bytes = int(os.environ.get("FLEXSAE_HIER_STAGE_MB", "4096")) << 20
+
+
+def set_hier_stage_bytes(nbytes: int) -> None:
+    """Upper bound (bytes) on what the fused training step keeps alive from forward to backward.
+    Calls whose contributions do not fit run the separate forward and sliced backward instead;
+    0 switches the fused step off for every shape."""
+    global _hier_stage_bytes
+    _hier_stage_bytes = int(nbytes)
 
 
 @torch.library.custom_op("flexsae_amd::hier_bwd", mutates_args=())
@@ -253,6 +268,130 @@ def _setup_context(ctx, inputs, output):
     _, resid = output
     ctx.save_for_backward(indices, weight, vals, resid)
     ctx.leaf_dtypes = (vals.dtype, bias.dtype, target.dtype)
+    ctx.set_materialize_grads(False)  # no zero-filled gradient for the saved residual
+
+
+# Training-step fusion: when gradients will be needed, compute loss and (unit-gradient) gradients
+# in one pass that gathers the weight rows once; the backward then only scales by grad_out.
+_fused_training = os.environ.get("FLEXSAE_FUSED_TRAINING", "1") not in ("", "0")
+
+
+def set_fused_training(enabled: bool) -> None:
+    """Enable/disable the fused forward + reverse walk of the hierarchical loss (default on).
+
+    It is used when gradients are required AND the stage budget (``set_hier_stage_bytes``)
+    can hold all per-pair contributions at once (B*K*D elements): the weight rows are then
+    gathered once per training step instead of twice, the contributions wait in the scratch and
+    the backward only runs the segment reduction, scaled by the upstream gradient.  Code that
+    evaluates the loss with gradients enabled but never calls ``backward()`` pays for the reverse
+    walk anyway: switch it off there or use ``torch.no_grad()``."""
+    global _fused_training
+    _fused_training = bool(enabled)
+
+
+def _train_supported(weight: Tensor, K: int) -> bool:
+    D = weight.shape[1]
+    return D % 4 == 0 and K <= (64 if weight.dtype == torch.float32 else 128)
+
+
+def _stage_fits(indices: Tensor, weight: Tensor) -> bool:
+    """The fused pass keeps one contribution per (b, k, d) alive until the backward; it is taken
+    only when the stage budget covers that."""
+    B, K = indices.shape
+    D = weight.shape[1]
+    p_size = 2 if weight.dtype == torch.bfloat16 else 4
+    return B * K * (-(-D // 256) * 256) * p_size <= _hier_stage_bytes
+
+
+def _single_slice_workspace_bytes(lib, shape, D: int) -> int:
+    return lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), D)
+
+
+@torch.library.custom_op("flexsae_amd::hier_train", mutates_args=())
+def hier_train(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
+               target: Tensor) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Fused forward + reverse walk with the segment reduction deferred.
+
+    Returns (loss, dvals, dbias, stage): dvals/dbias for a unit upstream gradient, and the
+    workspace holding the pair list and all per-pair contributions, from which
+    ``hier_finish`` produces dW with the upstream gradient folded in."""
+    B, K, F, D = _validate(indices, weight, vals, bias, target)
+    lib = _lib.load()
+    indices, weight, vals, bias, target = (t.contiguous() for t in (indices, weight, vals, bias, target))
+    dev = weight.device
+    with torch.cuda.device(dev):
+        shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
+        ws_bytes = _single_slice_workspace_bytes(lib, shape, D)
+        stage = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
+        dbias = torch.empty((D,), dtype=torch.float32, device=dev)
+        flag = _flag_for(dev)
+        rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
+                                      _ptr(target), _ptr(loss), None, _DTYPES[weight.dtype], _ptr(dvals),
+                                      _ptr(dbias), _ptr(stage), ws_bytes, _lib.BWD_SWEEP_ONLY, _ptr(flag),
+                                      _stream())
+        _lib.check(rc, "flexsae_hier_fwd_bwd")
+        if _check_indices:
+            check_index_flag(dev)
+    return loss, dvals, dbias, stage
+
+
+@hier_train.register_fake
+def _(indices, weight, vals, bias, target):
+    B, K = indices.shape
+    F, D = weight.shape
+    shape = _shape(int(B), int(K), int(F), int(D), weight, vals, bias.dtype, target.dtype)
+    ws_bytes = _single_slice_workspace_bytes(_lib.load(), shape, int(D))  # host-side size query
+    return (weight.new_empty((), dtype=torch.float32), vals.new_empty(vals.shape, dtype=torch.float32),
+            weight.new_empty((weight.shape[1],), dtype=torch.float32),
+            weight.new_empty((ws_bytes,), dtype=torch.uint8))
+
+
+@torch.library.custom_op("flexsae_amd::hier_finish", mutates_args=())
+def hier_finish(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor, stage: Tensor) -> Tensor:
+    """dW = grad_out * (segment sums of the contributions staged by ``hier_train``)."""
+    lib = _lib.load()
+    B, K = indices.shape
+    F, D = weight.shape
+    dev = weight.device
+    with torch.cuda.device(dev):
+        g = _grad_scalar(grad_out, dev)
+        shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
+        dW = torch.empty((F, D), dtype=weight.dtype, device=dev)
+        flags = _lib.BWD_REUSE_PAIR_LIST | _lib.BWD_REDUCE_ONLY | _lib.BWD_SCALE_BY_GRAD_OUT
+        rc = lib.flexsae_hier_bwd(ctypes.byref(shape), None, None, None, None, _ptr(g), _ptr(dW),
+                                  _DTYPES[weight.dtype], None, None, _ptr(stage), stage.numel(), flags, None,
+                                  _stream())
+        _lib.check(rc, "flexsae_hier_bwd (deferred reduction)")
+    return dW
+
+
+@hier_finish.register_fake
+def _(grad_out, indices, weight, vals, stage):
+    return torch.empty_like(weight)
+
+
+def _train_setup_context(ctx, inputs, output):
+    indices, weight, vals, bias, _ = inputs
+    _, dvals, dbias, stage = output
+    ctx.save_for_backward(indices, weight, vals, dvals, dbias, stage)
+    ctx.leaf_dtypes = (vals.dtype, bias.dtype)
+    # unused outputs (the stage above all) must not get zero-filled gradient tensors
+    ctx.set_materialize_grads(False)
+
+
+def _train_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_stage):
+    indices, weight, vals, dvals, dbias, stage = ctx.saved_tensors
+    if grad_loss is None:
+        return None, None, None, None, None
+    g = grad_loss.to(torch.float32)
+    vdt, bdt = ctx.leaf_dtypes
+    dW = hier_finish(g, indices, weight, vals, stage)
+    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None
+
+
+hier_train.register_autograd(_train_backward, setup_context=_train_setup_context)
 
 
 def _hier_backward(ctx, grad_loss, grad_resid):
@@ -289,6 +428,10 @@ def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, 
 
     Same name, argument order and meaning as the reference entry point
     (torch-ext/flex_sae/hierarchical_kernels.py:302-309); the kernels underneath are HIP."""
+    needs_grad = torch.is_grad_enabled() and (weight.requires_grad or vals.requires_grad or bias.requires_grad)
+    if (needs_grad and _fused_training and weight.dim() == 2 and indices.dim() == 2
+            and _train_supported(weight, indices.shape[1]) and _stage_fits(indices, weight)):
+        return hier_train(indices, weight, vals, bias, target)[0]
     return hier_fwd(indices, weight, vals, bias, target)[0]
 
 

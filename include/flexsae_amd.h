@@ -57,8 +57,14 @@ enum {
   /* flexsae_hier_bwd only: */
   FLEXSAE_BWD_REUSE_PAIR_LIST = 2,   /* the workspace still holds the pair list of a previous   */
                                      /* call with the same indices and shape: do not rebuild it */
-  FLEXSAE_BWD_SWEEP_ONLY = 4,        /* measurement aid: run only the sweep kernels             */
-  FLEXSAE_BWD_REDUCE_ONLY = 8        /* measurement aid: run only the segment reductions        */
+  FLEXSAE_BWD_SWEEP_ONLY = 4,        /* run only the sweep kernels (contributions stay in the   */
+                                     /* workspace; meaningful when one slice covers all of D)   */
+  FLEXSAE_BWD_REDUCE_ONLY = 8,       /* run only the segment reductions on the contributions    */
+                                     /* already in the workspace; with REUSE_PAIR_LIST and a    */
+                                     /* single-slice workspace only grad_out, dW and workspace  */
+                                     /* are read (the rest may be NULL): the deferred reduction */
+  FLEXSAE_BWD_SCALE_BY_GRAD_OUT = 16 /* deferred reduction only: the contributions were made    */
+                                     /* for a unit upstream gradient; multiply dW by grad_out[0]*/
 };
 
 /* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^31; B*K < 2^32. */
@@ -125,6 +131,42 @@ int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const v
                      const void *vals, const float *resid, const float *grad_out, void *dW,
                      int dW_dtype, float *dvals, float *dbias, void *workspace,
                      size_t workspace_bytes, int flags, int *status_flag, void *stream);
+
+/*
+ * HierarchicalTopK training step: forward AND backward in one pass over the gathered rows.
+ * The sweep kernel of flexsae_hier_bwd is replaced by a kernel that gathers each row piece
+ * once, keeps the K pieces of a (row, 128-column tile) in registers, walks them forward (loss)
+ * and then backward (contributions, dvals), so the weight rows are gathered once per step
+ * instead of twice.  The gradients returned are those of a UNIT upstream gradient; multiply by
+ * the real one afterwards (flexsae_scale for dW; dvals/dbias are small).  Same workspace, same
+ * slicing and the same segment reduction as flexsae_hier_bwd (use
+ * flexsae_hier_bwd_workspace_bytes).
+ * Supported when D % 4 == 0 and K <= 128 (bf16/fp16 weights) or K <= 64 (fp32 weights):
+ * flexsae_hier_fwd_bwd_supported() tells; otherwise FLEXSAE_ERR_UNSUPPORTED (use
+ * flexsae_hier_fwd + flexsae_hier_bwd).
+ * replaces: the forward and backward kernels and launchers together
+ *           (hierarchical_kernels.py:12-187, 190-270), for the loss.backward() pattern of
+ *           the reference's training loop (reference example.py:76-77).
+ * out: loss[1]; dW[F,D] in dW_dtype; dvals[B,K] fp32; dbias[D] fp32 -- for grad_out = 1.
+ * Deferred reduction: with FLEXSAE_BWD_SWEEP_ONLY in `flags` (and a workspace wide enough for a
+ * single slice, else FLEXSAE_ERR_WORKSPACE) the segment reduction is left out and dW is not
+ * touched (may be NULL); a later flexsae_hier_bwd on the same workspace with
+ * FLEXSAE_BWD_REUSE_PAIR_LIST | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SCALE_BY_GRAD_OUT finishes dW
+ * with the upstream gradient folded in, so no separate scaling pass over dW is needed.  The
+ * price is that the workspace (B*K*D contributions) must stay alive in between.
+ */
+int flexsae_hier_fwd_bwd_supported(const flexsae_shape *shape);
+int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
+                         const void *vals, const void *bias, const void *target, float *loss,
+                         void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
+                         size_t workspace_bytes, int flags, int *status_flag, void *stream);
+
+/*
+ * dst[n] = src[n] * scale[0]  (same dtype in and out; `scale` is a device fp32 scalar).
+ * replaces: the dW.mul_(grad) pass of HierarchicalSAELossFunction.backward
+ *           (hierarchical_kernels.py:294-297), needed only after flexsae_hier_fwd_bwd.
+ */
+int flexsae_scale(void *dst, const void *src, int dtype, int64_t n, const float *scale, void *stream);
 
 /*
  * HierarchicalTopK backward, single-pass fallback that needs no workspace: the same reverse

@@ -58,6 +58,31 @@ def hier_backward(indices, weight, vals, resid, grad_out, flag=None, slice_cols=
     return rc, dW, dv, db
 
 
+def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_dtype=torch.float32):
+    """Fused forward+backward for a unit upstream gradient -> (rc, loss, dW, dvals, dbias)."""
+    lib = _lib.load()
+    sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
+    dev = weight.device
+    loss = torch.full((1,), float("nan"), dtype=torch.float32, device=dev)
+    dW = torch.full((sh.F, sh.D), float("nan"), dtype=dw_dtype, device=dev)
+    dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
+    db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
+    nbytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(bias), ptr(target),
+                                  ptr(loss), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, 0,
+                                  ptr(flag), stream())
+    return rc, loss, dW, dv, db
+
+
+def scale(src, g):
+    lib = _lib.load()
+    dst = torch.full_like(src, float("nan"))
+    gt = torch.tensor([g], dtype=torch.float32, device=src.device)
+    rc = lib.flexsae_scale(ptr(dst), ptr(src), DT[src.dtype], src.numel(), ptr(gt), stream())
+    return rc, dst
+
+
 def hier_backward_atomic(indices, weight, vals, resid, grad_out, flag=None, prezeroed=False):
     """Atomic fallback -> (rc, dW_acc fp32, dvals fp32, dbias fp32)."""
     lib = _lib.load()

@@ -76,6 +76,84 @@ def test_reference_matrix(mode, B, K, F, D, dtype):
     _check_against_oracle(mode, args, dtype, grad_out, got)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("B,K,F,D", PARAMS[::3])
+def test_reference_matrix_without_fused_training(B, K, F, D, dtype):
+    """The hierarchical loss takes the fused forward+backward pass by default when gradients are
+    required; this runs every third shape through the separate forward / backward kernels."""
+    _announce("matrix unfused", B, K, F, D, dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype)
+    flex.set_fused_training(False)
+    try:
+        got = _run_op("hier", args, -0.6)
+    finally:
+        flex.set_fused_training(True)
+    _check_against_oracle("hier", args, dtype, -0.6, got)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(48, 32, 200, 768), (7, 5, 300, 260), (33, 128, 64, 2304), (16, 64, 9, 132),
+                                   (5, 100, 40, 512), (64, 16, 1000, 4)])
+def test_training_step_entry_point(shape, dtype):
+    """flexsae_hier_fwd_bwd through the C-ABI: loss and unit-gradient gradients in one pass, for
+    K that are not powers of two, D that are not whole tiles, hot latents (F tiny)."""
+    B, K, F, D = shape
+    _announce("train abi", shape, dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=41)
+    idx, W, v, b, t = _to_dev(args)
+    rc, loss, dW, dv, db = abi.hier_train(idx, W, v, b, t)
+    torch.cuda.synchronize()
+    if dtype == torch.float32 and K > 64:
+        assert rc == -2  # FLEXSAE_ERR_UNSUPPORTED: fp32 rows of K > 64 do not fit in registers
+        return
+    assert rc == 0
+    L, rW, rv, rb = oracle.loss_grads(oracle.HIER, *args, grad_out=1.0)
+    tol_loss, _ = REL_TOL[dtype]
+    assert abs(loss.item() - L) <= tol_loss * abs(L)
+    assert rel_err(dW.cpu(), rW) < (4e-3 if dtype == torch.bfloat16 else 1e-4)
+    assert rel_err(dv.cpu(), rv) < 1e-4 and rel_err(db.cpu(), rb) < 1e-4
+    # bit-identical dW for any slice width, and equal to the two-kernel path's
+    rc2, _, dW2, _, _ = abi.hier_train(idx, W, v, b, t, slice_cols=1 << 20)
+    assert rc2 == 0 and torch.equal(dW, dW2)
+    rc3, loss3, resid = abi.forward("hier", idx, W, v, b, t)
+    rc4, dW4, dv4, db4 = abi.hier_backward(idx, W, v, resid, 1.0)
+    assert rc3 == rc4 == 0
+    assert abs(loss.item() - loss3.item()) <= 2e-6 * abs(L)
+    assert rel_err(dW.cpu(), dW4.cpu()) < (4e-3 if dtype == torch.bfloat16 else 2e-5)
+    assert rel_err(dv.cpu(), dv4.cpu()) < 2e-5
+
+
+def test_training_step_unsupported_shapes_and_scale():
+    idx, W, v, b, t = _to_dev(make_inputs(8, 8, 32, 6, seed=3))  # D % 4 != 0
+    rc, *_ = abi.hier_train(idx, W, v, b, t)
+    assert rc == -2
+    idx, W, v, b, t = _to_dev(make_inputs(4, 130, 32, 64, dtype=torch.bfloat16, seed=3))  # K > 128
+    rc, *_ = abi.hier_train(idx, W, v, b, t)
+    assert rc == -2
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        x = torch.randn(1003, device=DEV).to(dt)
+        rc, y = abi.scale(x, -2.5)
+        assert rc == 0 and torch.equal(y, (x.float() * -2.5).to(dt))
+
+
+def test_fused_training_backward_twice_and_no_grad():
+    """retain_graph + two backward calls accumulate correctly; no_grad / non-leaf-free inputs take
+    the forward-only kernel."""
+    args = make_inputs(32, 16, 100, 512, dtype=torch.bfloat16, seed=8)
+    idx, W, v, b, t = _to_dev(args)
+    W.requires_grad_()
+    loss = flex.triton_hierarchical_sae_loss(idx, W, v, b, t)
+    loss.backward(torch.tensor(2.0, device=DEV), retain_graph=True)
+    g1 = W.grad.clone()
+    loss.backward(torch.tensor(-0.5, device=DEV))
+    L, rW, _, _ = oracle.loss_grads(oracle.HIER, *args, grad_out=1.5)
+    assert rel_err(W.grad.float().cpu(), rW) < 2e-2
+    assert rel_err(g1.float().cpu(), rW * (2.0 / 1.5)) < 1e-2
+    with torch.no_grad():
+        l2 = flex.triton_hierarchical_sae_loss(idx, W, v, b, t)
+    assert not l2.requires_grad and abs(l2.item() - loss.item()) <= 2e-6 * abs(L)
+
+
 @pytest.mark.parametrize("mode", ["hier", "topk"])
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (3, 5, 7, 9), (5, 3, 11, 70), (2, 65, 40, 130),
                                    (7, 130, 300, 200), (4, 24, 50, 1000), (33, 12, 17, 2304)])
@@ -271,13 +349,16 @@ def test_hier_dw_is_reproducible_bit_for_bit():
 
 @pytest.mark.parametrize("mode", ["segment", "atomic"])
 def test_hier_backward_variants_through_the_op(mode):
-    """Both backward implementations behind the public op (scratch budget 0 = atomic fallback)."""
+    """Both stand-alone backward implementations behind the public op (scratch budget 0 = atomic
+    fallback, 1 MiB = several slices), reached because the stage budget is too small to fuse."""
     args = make_inputs(48, 32, 200, 768, dtype=torch.bfloat16, seed=13)
     flex.set_hier_scratch_bytes(0 if mode == "atomic" else 1 << 20)
+    flex.set_hier_stage_bytes(1 << 20)
     try:
         got = _run_op("hier", args, 1.5)
     finally:
         flex.set_hier_scratch_bytes(256 << 20)
+        flex.set_hier_stage_bytes(4096 << 20)
     _check_against_oracle("hier", args, torch.bfloat16, 1.5, got)
 
 
@@ -355,9 +436,11 @@ def test_opcheck_and_compile(mode):
     W.requires_grad_()
     v.requires_grad_()
     b.requires_grad_()
-    op = torch.ops.flexsae_amd.hier_fwd if mode == "hier" else torch.ops.flexsae_amd.topk_fwd
-    torch.library.opcheck(op, (idx, W, v, b, t),
-                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+    ops_ = ([torch.ops.flexsae_amd.hier_fwd, torch.ops.flexsae_amd.hier_train] if mode == "hier"
+            else [torch.ops.flexsae_amd.topk_fwd])
+    for op in ops_:
+        torch.library.opcheck(op, (idx, W, v, b, t),
+                              test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
     eager = FUSED[mode](idx, W, v, b, t)
     compiled = torch.compile(lambda *a: FUSED[mode](*a) * 2.0, fullgraph=True, backend="aot_eager")(idx, W, v, b, t)
     assert abs(compiled.item() - 2.0 * eager.item()) <= 1e-6 * abs(eager.item())
