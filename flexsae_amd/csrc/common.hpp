@@ -97,24 +97,29 @@ __device__ __forceinline__ void load_vec(const void *base, int64_t off, float (&
   }
 }
 
-template <typename T, int VEC>
+// NT: non-temporal (streaming) store, for data that is written once and not read again soon,
+// so that it does not push reusable lines out of the L2.
+template <typename T, int VEC, bool NT = false>
 __device__ __forceinline__ void store_vec(void *base, int64_t off, const float (&x)[VEC]) {
   using S = typename Traits<T>::store_t;
   S *p = static_cast<S *>(base) + off;
+  auto put = [](auto *dst, auto v) {
+    if constexpr (NT) __builtin_nontemporal_store(v, dst); else *dst = v;
+  };
   if constexpr (Traits<T>::dtype == FLEXSAE_BF16 && VEC == 2) {
-    *reinterpret_cast<uint32_t *>(p) = f32x2_to_bf16x2_bits(x[0], x[1]);
+    put(reinterpret_cast<uint32_t *>(p), f32x2_to_bf16x2_bits(x[0], x[1]));
   } else if constexpr (Traits<T>::dtype == FLEXSAE_BF16 && VEC > 2) {
     vec_t<uint32_t, VEC / 2> v;
 #pragma unroll
     for (int i = 0; i < VEC / 2; ++i) v[i] = f32x2_to_bf16x2_bits(x[2 * i], x[2 * i + 1]);
-    *reinterpret_cast<vec_t<uint32_t, VEC / 2> *>(p) = v;
+    put(reinterpret_cast<vec_t<uint32_t, VEC / 2> *>(p), v);
   } else if constexpr (VEC == 1) {
-    *p = Traits<T>::down(x[0]);
+    put(p, Traits<T>::down(x[0]));
   } else {
     vec_t<S, VEC> v;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) v[i] = Traits<T>::down(x[i]);
-    *reinterpret_cast<vec_t<S, VEC> *>(p) = v;
+    put(reinterpret_cast<vec_t<S, VEC> *>(p), v);
   }
 }
 
@@ -146,6 +151,8 @@ __device__ __forceinline__ float dpp_move(float v) {
       __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
 }
 
+__device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }
+
 // Sum over the 64 lanes of the wavefront using DPP moves only (no LDS traffic).
 // The total is valid in lane 63; use wave_sum_bcast() to have it in every lane.
 __device__ __forceinline__ float wave_sum_lane63(float v) {
@@ -163,7 +170,98 @@ __device__ __forceinline__ float wave_sum_bcast(float v) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
-__device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) & (kWave - 1); }
+// Sum over the 64 lanes of eight values per lane at once: returns, in lane L, the wave-wide
+// total of d[L & 7].  Three exchange stages inside each group of 8 lanes halve the number of
+// live values while doubling the lanes summed (partner L^7, then L^2, then L^1: together they
+// generate the whole group), then three stages add the eight groups (L^8 by a row rotation,
+// L^16 and L^32 by lane permutes).  About 3.5 VALU operations per value instead of 12.
+__device__ __forceinline__ float wave_sum8_transposed(const float (&d)[8]) {
+  const int lane = lane_id();
+  const bool b2 = (lane & 4) != 0, b1 = (lane & 2) != 0, b0 = (lane & 1) != 0;
+  float r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float keep = b2 ? d[i + 4] : d[i];
+    const float give = b2 ? d[i] : d[i + 4];
+    r[i] = keep + dpp_move<0x141>(give);  // row_half_mirror: lane ^ 7
+  }
+  float q[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float keep = b1 ? r[i + 2] : r[i];
+    const float give = b1 ? r[i] : r[i + 2];
+    q[i] = keep + dpp_move<0x4E>(give);  // quad_perm [2,3,0,1]: lane ^ 2
+  }
+  const float keep = b0 ? q[1] : q[0];
+  const float give = b0 ? q[0] : q[1];
+  float z = keep + dpp_move<0xB1>(give);  // quad_perm [1,0,3,2]: lane ^ 1
+  z += dpp_move<0x128>(z);                // row_ror:8 within the 16-lane row: lane ^ 8
+  z += __shfl_xor(z, 16, kWave);
+  z += __shfl_xor(z, 32, kWave);
+  return z;
+}
+
+// VEC consecutive elements as stored (no conversion): lets a kernel keep many loads in flight
+// in few registers and convert at the point of use.
+template <typename T, int VEC>
+using raw_vec_t = vec_t<typename Traits<T>::store_t, VEC>;
+
+template <typename T, int VEC, bool NT = false>
+__device__ __forceinline__ raw_vec_t<T, VEC> load_raw(const void *base, int64_t off) {
+  using S = typename Traits<T>::store_t;
+  const raw_vec_t<T, VEC> *p = reinterpret_cast<const raw_vec_t<T, VEC> *>(static_cast<const S *>(base) + off);
+  if constexpr (NT) return __builtin_nontemporal_load(p);  // read once: do not keep it in the L2
+  else return *p;
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void unpack_raw(const raw_vec_t<T, VEC> &v, float (&o)[VEC]) {
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) o[i] = Traits<T>::up(v[i]);
+}
+
+
+// Row gathers through a buffer descriptor: the lane's byte offset travels in a vector register,
+// the (uniform) row offset in a scalar one, so a gather costs no vector ALU work for addressing;
+// reads beyond `bytes` return zeros.  The matrix must be smaller than 4 GiB.
+struct GatherSource {
+  __amdgpu_buffer_rsrc_t rsrc;
+};
+__device__ __forceinline__ GatherSource make_gather_source(const void *base, uint32_t bytes) {
+  GatherSource g;
+  g.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(bytes), 0x00020000);
+  return g;
+}
+template <typename T, int VEC>
+__device__ __forceinline__ raw_vec_t<T, VEC> gather_raw(const GatherSource &g, uint32_t lane_bytes,
+                                                        uint32_t row_bytes_offset) {
+  constexpr int kBytes = VEC * static_cast<int>(sizeof(typename Traits<T>::store_t));
+  raw_vec_t<T, VEC> out;
+  if constexpr (kBytes == 2) {
+    const uint16_t v = __builtin_amdgcn_raw_buffer_load_b16(g.rsrc, lane_bytes, row_bytes_offset, 0);
+    __builtin_memcpy(&out, &v, 2);
+  } else if constexpr (kBytes == 4) {
+    const uint32_t v = __builtin_amdgcn_raw_buffer_load_b32(g.rsrc, lane_bytes, row_bytes_offset, 0);
+    __builtin_memcpy(&out, &v, 4);
+  } else if constexpr (kBytes == 8) {
+    const vec_t<uint32_t, 2> v = __builtin_amdgcn_raw_buffer_load_b64(g.rsrc, lane_bytes, row_bytes_offset, 0);
+    __builtin_memcpy(&out, &v, 8);
+  } else {
+    static_assert(kBytes == 16, "gathers are 2 to 16 bytes per lane");
+    const vec_t<uint32_t, 4> v = __builtin_amdgcn_raw_buffer_load_b128(g.rsrc, lane_bytes, row_bytes_offset, 0);
+    __builtin_memcpy(&out, &v, 16);
+  }
+  return out;
+}
+
+// acc + a.lo*b.lo + a.hi*b.hi on two packed bf16 pairs (one instruction on gfx950)
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  bf16x2 x, y;
+  __builtin_memcpy(&x, &a, 4);
+  __builtin_memcpy(&y, &b, 4);
+  return __builtin_amdgcn_fdot2_f32_bf16(x, y, acc, false);
+}
 
 // Wave index inside the block as a scalar (uniform) value, so that everything
 // derived from it is addressed through scalar registers.

@@ -26,6 +26,9 @@ using namespace flexsae;
 #ifndef FLEXSAE_TOPK_U
 #define FLEXSAE_TOPK_U 4
 #endif
+#ifndef FLEXSAE_TOPK_RESID16
+#define FLEXSAE_TOPK_RESID16 1
+#endif
 
 namespace {
 
@@ -454,7 +457,8 @@ struct TopkBwdPlan {
   int vec, tile;
   int64_t d_pad;
   size_t n_pairs, n_partial_rows;
-  size_t off_colsum, off_long_count, off_long_list, off_chunk, off_partial, fixed_bytes;
+  size_t off_colsum, off_long_count, off_long_list, off_chunk, off_resid16, off_dvpart, off_slotbv, off_partial, fixed_bytes;
+  bool resid16;  // gather a bf16 copy of the residual (bf16 weights): half the cache footprint
 };
 
 TopkBwdPlan plan_topk_bwd(const flexsae_shape *s) {
@@ -473,6 +477,15 @@ TopkBwdPlan plan_topk_bwd(const flexsae_shape *s) {
   off += round_up((p.n_pairs / 65 + 1) * 4, kAlign);
   p.off_chunk = off;
   off += round_up((p.n_pairs / 65 + 2) * 4, kAlign);
+  // The reference hands its backward the residual gradient in the weight dtype
+  // (topk_kernels.py:52,221); for bf16 weights the gathers here read a bf16 copy as well.
+  p.resid16 = FLEXSAE_TOPK_RESID16 && s->weight_dtype == FLEXSAE_BF16;
+  p.off_resid16 = off;
+  if (p.resid16) off += round_up(static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * 2, kAlign);
+  p.off_dvpart = off;  // per-tile shares of dvals: [d_pad / tile, B*K] fp32
+  off += round_up(static_cast<size_t>(p.d_pad / p.tile) * p.n_pairs * 4, kAlign);
+  p.off_slotbv = off;  // (batch row, val) of every pair in pair-list order
+  off += round_up(p.n_pairs * 8, kAlign);
   p.off_partial = off;
   p.fixed_bytes = off;
   return p;
@@ -482,68 +495,78 @@ size_t topk_bwd_bytes(const TopkBwdPlan &p, int64_t slice_w) {
   return p.fixed_bytes + round_up(p.n_partial_rows * static_cast<size_t>(slice_w) * 4, kAlign);
 }
 
-template <typename WT, typename GT, int VEC>
+template <typename WT, typename GT, typename RT, int VEC>
 void launch_topk_slices(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t slice_w,
                         const uint32_t *begin, const uint32_t *map, const void *weight,
-                        const void *vals, const float *resid, const float *grad_out, float coef,
+                        const void *vals, const void *resid, const float *grad_out, float coef,
                         void *dW, float *dvals, uint8_t *ws, hipStream_t st) {
   const uint32_t *long_count = reinterpret_cast<const uint32_t *>(ws + pl.off_long_count);
   const uint32_t *long_list = reinterpret_cast<const uint32_t *>(ws + pl.off_long_list);
   const uint32_t *chunk_begin = reinterpret_cast<const uint32_t *>(ws + pl.off_chunk);
   float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
+  float *dv_part = reinterpret_cast<float *>(ws + pl.off_dvpart);
+  const int64_t n_pairs = static_cast<int64_t>(pl.n_pairs);
   const int K = static_cast<int>(s->K), D = static_cast<int>(s->D), sw = static_cast<int>(slice_w);
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
-    const int64_t n_items = s->F * tps;
-    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock));
-    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, VEC, FLEXSAE_TOPK_U>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock), 0,
-                       st, begin, map, long_count, long_list, chunk_begin, weight, vals, s->vals_dtype, resid,
-                       grad_out, coef, dW, dvals, partial, n_items, kLongBlocks, tps, static_cast<int>(col0),
-                       sw, s->F, K, D);
+    const int64_t n_short_blocks = ceil_div(s->F * tps, static_cast<int64_t>(kWavesPerBlock));
+    const size_t resid_bytes =
+        static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * sizeof(typename Traits<RT>::store_t);
+    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, RT, VEC, FLEXSAE_TOPK_U>),
+                       dim3(kLongBlocks + static_cast<unsigned>(n_short_blocks)), dim3(kBlock), 0, st, begin, map,
+                       long_count, long_list, chunk_begin,
+                       reinterpret_cast<const vec_t<uint32_t, 2> *>(ws + pl.off_slotbv), weight, vals,
+                       s->vals_dtype, resid, grad_out, coef, dW, dv_part, n_pairs, partial, kLongBlocks, tps,
+                       static_cast<int>(col0), sw, s->F, K, D, static_cast<uint32_t>(resid_bytes));
     hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
                        long_count, long_list, chunk_begin, partial, dW, static_cast<const float *>(nullptr), tps,
                        static_cast<int>(col0), sw, D);
   }
 }
 
-template <typename WT, int VEC>
+template <typename WT, typename RT, int VEC>
 void launch_topk_slices_g(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t slice_w,
                           const uint32_t *begin, const uint32_t *map, const void *weight,
-                          const void *vals, const float *resid, const float *grad_out, float coef,
+                          const void *vals, const void *resid, const float *grad_out, float coef,
                           void *dW, int dW_dtype, float *dvals, uint8_t *ws, hipStream_t st) {
   switch (dW_dtype) {
     case FLEXSAE_F32:
-      launch_topk_slices<WT, float, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef,
-                                         dW, dvals, ws, st);
+      launch_topk_slices<WT, float, RT, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out,
+                                             coef, dW, dvals, ws, st);
       break;
     case FLEXSAE_BF16:
-      launch_topk_slices<WT, bf16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef,
-                                          dW, dvals, ws, st);
+      launch_topk_slices<WT, bf16_t, RT, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out,
+                                              coef, dW, dvals, ws, st);
       break;
     default:
-      launch_topk_slices<WT, f16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef,
-                                         dW, dvals, ws, st);
+      launch_topk_slices<WT, f16_t, RT, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out,
+                                             coef, dW, dvals, ws, st);
   }
 }
 
+// `resid` is the fp32 residual, or its bf16 copy when the plan says so (bf16 weights only)
 template <int VEC>
 void launch_topk_slices_w(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t slice_w,
                           const uint32_t *begin, const uint32_t *map, const void *weight,
-                          const void *vals, const float *resid, const float *grad_out, float coef,
+                          const void *vals, const void *resid, const float *grad_out, float coef,
                           void *dW, int dW_dtype, float *dvals, uint8_t *ws, hipStream_t st) {
   switch (s->weight_dtype) {
     case FLEXSAE_F32:
-      launch_topk_slices_g<float, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW,
-                                       dW_dtype, dvals, ws, st);
+      launch_topk_slices_g<float, float, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out,
+                                              coef, dW, dW_dtype, dvals, ws, st);
       break;
     case FLEXSAE_BF16:
-      launch_topk_slices_g<bf16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW,
-                                        dW_dtype, dvals, ws, st);
+      if (pl.resid16)
+        launch_topk_slices_g<bf16_t, bf16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out,
+                                                  coef, dW, dW_dtype, dvals, ws, st);
+      else
+        launch_topk_slices_g<bf16_t, float, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out,
+                                                 coef, dW, dW_dtype, dvals, ws, st);
       break;
     default:
-      launch_topk_slices_g<f16_t, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW,
-                                       dW_dtype, dvals, ws, st);
+      launch_topk_slices_g<f16_t, float, VEC>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out,
+                                              coef, dW, dW_dtype, dvals, ws, st);
   }
 }
 
@@ -808,6 +831,8 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
   if (!begin || !map || !weight || !vals || !resid || !grad_out || !dW || !dvals || !dbias ||
       !valid_dtype(dW_dtype))
     return FLEXSAE_ERR_INVALID_ARGUMENT;
+  // the residual rows are gathered through a 32-bit buffer descriptor
+  if (static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * 4 > 0xffffffffull) return FLEXSAE_ERR_UNSUPPORTED;
   const TopkBwdPlan pl = plan_topk_bwd(s);
   if (!aligned(begin, 4) || !aligned(map, 4) || !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
       !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.vec * 4) || !aligned(grad_out, 4) ||
@@ -820,7 +845,7 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
     slice_w += pl.tile;
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint8_t *ws = static_cast<uint8_t *>(workspace);
-  if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) zero_f32(dvals, s->B * s->K, st);
+  (void)flags;  // every output element is written exactly once: nothing needs a zero-fill
   // latents with more than 64 pairs and their chunk table
   uint32_t *long_count = reinterpret_cast<uint32_t *>(ws + pl.off_long_count);
   uint32_t *long_list = reinterpret_cast<uint32_t *>(ws + pl.off_long_list);
@@ -831,16 +856,30 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
                      reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
   const float coef =
       static_cast<float>(2.0 / (static_cast<double>(s->B) * static_cast<double>(s->D)));
-  if (pl.vec == 4) {
-    launch_topk_slices_w<4>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                            dvals, ws, st);
-  } else if (pl.vec == 2) {
-    launch_topk_slices_w<2>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                            dvals, ws, st);
-  } else {
-    launch_topk_slices_w<1>(s, pl, slice_w, begin, map, weight, vals, resid, grad_out, coef, dW, dW_dtype,
-                            dvals, ws, st);
+  hipLaunchKernelGGL(topk_slot_records_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map, vals,
+                     s->vals_dtype, s->B * s->K, static_cast<int>(s->K),
+                     reinterpret_cast<vec_t<uint32_t, 2> *>(ws + pl.off_slotbv));
+  const void *gather_src = resid;
+  if (pl.resid16) {
+    void *r16 = ws + pl.off_resid16;
+    const int64_t n = s->B * s->D;
+    hipLaunchKernelGGL(cast_from_f32_kernel<bf16_t>, dim3(grid_for(ceil_div(n, 4), 256, 1 << 16)), dim3(256), 0,
+                       st, r16, resid, n);
+    gather_src = r16;
   }
+  if (pl.vec == 4) {
+    launch_topk_slices_w<4>(s, pl, slice_w, begin, map, weight, vals, gather_src, grad_out, coef, dW,
+                            dW_dtype, dvals, ws, st);
+  } else if (pl.vec == 2) {
+    launch_topk_slices_w<2>(s, pl, slice_w, begin, map, weight, vals, gather_src, grad_out, coef, dW,
+                            dW_dtype, dvals, ws, st);
+  } else {
+    launch_topk_slices_w<1>(s, pl, slice_w, begin, map, weight, vals, gather_src, grad_out, coef, dW,
+                            dW_dtype, dvals, ws, st);
+  }
+  hipLaunchKernelGGL(topk_dvals_finalize_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
+                     reinterpret_cast<const float *>(ws + pl.off_dvpart), static_cast<int>(pl.d_pad / pl.tile),
+                     s->B * s->K, dvals);
   rc = launch_status();
   if (rc != FLEXSAE_OK) return rc;
   // dbias = coef * grad_out * column sums of resid, in a fixed order

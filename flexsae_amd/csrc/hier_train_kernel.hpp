@@ -37,37 +37,6 @@ struct RowPiece2<f16_t> {
   static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
 };
 
-// Sum over the 64 lanes of eight values per lane at once: returns, in lane L, the wave-wide
-// total of d[L & 7].  Three exchange stages inside each group of 8 lanes halve the number of
-// live values while doubling the lanes summed (partner L^7, then L^2, then L^1: together they
-// generate the whole group), then three stages add the eight groups (L^8 by a row rotation,
-// L^16 and L^32 by lane permutes).  About 3.5 VALU operations per value instead of 12.
-__device__ __forceinline__ float wave_sum8_transposed(const float (&d)[8]) {
-  const int lane = lane_id();
-  const bool b2 = (lane & 4) != 0, b1 = (lane & 2) != 0, b0 = (lane & 1) != 0;
-  float r[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float keep = b2 ? d[i + 4] : d[i];
-    const float give = b2 ? d[i] : d[i + 4];
-    r[i] = keep + dpp_move<0x141>(give);  // row_half_mirror: lane ^ 7
-  }
-  float q[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const float keep = b1 ? r[i + 2] : r[i];
-    const float give = b1 ? r[i] : r[i + 2];
-    q[i] = keep + dpp_move<0x4E>(give);  // quad_perm [2,3,0,1]: lane ^ 2
-  }
-  const float keep = b0 ? q[1] : q[0];
-  const float give = b0 ? q[0] : q[1];
-  float z = keep + dpp_move<0xB1>(give);  // quad_perm [1,0,3,2]: lane ^ 1
-  z += dpp_move<0x128>(z);                // row_ror:8 within the 16-lane row: lane ^ 8
-  z += __shfl_xor(z, 16, kWave);
-  z += __shfl_xor(z, 32, kWave);
-  return z;
-}
-
 // One wavefront per (tile of the slice, row b), tile-major; a tile is 128 columns and lane l owns
 // columns 2l, 2l+1.  The wavefront issues the gathers of all K row pieces at once (the memory
 // pipeline keeps up to 63 of them in flight per wavefront, so a few wavefronts per SIMD cover the

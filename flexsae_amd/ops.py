@@ -243,8 +243,9 @@ def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
         dW = torch.empty_like(weight)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
-        # the slice width only sizes the partial sums of hot latents: 64 MiB of them is plenty
-        slice_cols = max(1, (64 << 20) // max(1, (B * K // 32) * 4))
+        # the slice width only sizes the partial sums of hot latents; one launch over all of D is
+        # fastest, so allow them 256 MiB before slicing
+        slice_cols = max(1, (256 << 20) // max(1, (B * K // 32) * 4))
         bws_bytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
         bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
         rc = lib.flexsae_topk_bwd(ctypes.byref(shape), _ptr(begin), _ptr(pair_map), _ptr(weight), _ptr(vals),

@@ -203,8 +203,13 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
  *           (topk_kernels.py:97-137, 165-184, 220-223)
  * in : begin/map from flexsae_csr_build; resid from flexsae_topk_fwd; grad_out device scalar.
  * out: dW[F,D] written once in `dW_dtype` (every row, zeros for unused latents);
- *      dvals[B,K] fp32 (zero-filled here unless FLEXSAE_BWD_OUTPUTS_PREZEROED) and
- *      dbias[D] fp32 (column sums in a fixed order: deterministic).
+ *      dvals[B,K] fp32, every element written once (per-tile shares added in tile order);
+ *      dbias[D] fp32 (column sums in a fixed order).  All three are bit-reproducible;
+ *      `flags` is accepted for symmetry and ignored (nothing needs a zero-fill).
+ * With bf16 weights the residual rows are gathered from a bf16 copy made in the workspace: the
+ * reference's backward likewise receives the residual gradient in the weight dtype
+ * (topk_kernels.py:52 makes the bag output weight-typed, so autograd casts its gradient).
+ * Limit: B*D*4 bytes < 4 GiB (FLEXSAE_ERR_UNSUPPORTED beyond), the gathers use 32-bit offsets.
  */
 int flexsae_topk_bwd(const flexsae_shape *shape, const uint32_t *begin, const uint32_t *map,
                      const void *weight, const void *vals, const float *resid,
@@ -215,7 +220,9 @@ int flexsae_topk_bwd(const flexsae_shape *shape, const uint32_t *begin, const ui
  * Bytes of workspace flexsae_topk_bwd needs to process `slice_cols` columns of D per pass
  * (rounded to whole tiles, capped at D; <= 0 asks for the minimum).  The slice width only
  * sizes the fp32 partial sums of latents with more than 64 pairs (hot latents are cut into
- * 64-pair chunks that are reduced by separate wavefronts and then combined in a fixed order).
+ * 64-pair chunks that are reduced by separate wavefronts and then combined in a fixed order);
+ * the fixed part holds the per-pair records, the per-tile dvals shares (D/256 x B*K fp32) and,
+ * for bf16 weights, the bf16 residual copy.
  */
 size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slice_cols);
 

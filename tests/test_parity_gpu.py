@@ -246,10 +246,11 @@ def test_c_abi_direct(mode, dtype):
     L, rW, rv, rb = oracle.loss_grads(MODES[mode], *args, grad_out=0.7)
     tol_loss, _ = REL_TOL[dtype]
     assert abs(loss.item() - L) <= tol_loss * abs(L)
-    # outputs here are fp32 whatever the input dtype, so the fp32 bar applies to the arithmetic
-    # (except that the two-phase hierarchical backward stores bf16 contributions for bf16 weights)
-    assert rel_err(dW.cpu(), rW) < (4e-3 if (mode == "hier" and dtype == torch.bfloat16) else 1e-4)
-    assert rel_err(dv.cpu(), rv) < 1e-4
+    # outputs here are fp32 whatever the input dtype, so the fp32 bar applies to the arithmetic,
+    # except that for bf16 weights the two-phase hierarchical backward stores bf16 contributions
+    # and the TopK backward gathers a bf16 copy of the residual (as the reference's does)
+    assert rel_err(dW.cpu(), rW) < (4e-3 if dtype == torch.bfloat16 else 1e-4)
+    assert rel_err(dv.cpu(), rv) < (4e-3 if (mode == "topk" and dtype == torch.bfloat16) else 1e-4)
     assert rel_err(db.cpu(), rb) < 1e-4
     # resid is r_{K-1} - target
     rW0 = W.float().cpu()[idx.cpu()] * v.float().cpu().unsqueeze(-1)
@@ -320,9 +321,10 @@ def test_topk_slice_width_does_not_change_the_result(shape, dtype):
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[1][0], outs[2][0])
     assert torch.equal(outs[0][2], outs[1][2])  # dbias: fixed-order column sums
     L, rW, rv, rb = oracle.loss_grads(oracle.TOPK, *args, grad_out=0.9)
-    assert rel_err(outs[0][0].cpu(), rW) < 1e-4
+    tol = 4e-3 if dtype == torch.bfloat16 else 1e-4  # bf16 weights: bf16 copy of the residual
+    assert rel_err(outs[0][0].cpu(), rW) < tol
     for _, dv, db in outs:
-        assert rel_err(dv.cpu(), rv) < 1e-4 and rel_err(db.cpu(), rb) < 1e-4
+        assert rel_err(dv.cpu(), rv) < tol and rel_err(db.cpu(), rb) < 1e-4
 
 
 @pytest.mark.parametrize("mode", ["hier", "topk"])
