@@ -254,6 +254,37 @@ __device__ __forceinline__ raw_vec_t<T, VEC> gather_raw(const GatherSource &g, u
   return out;
 }
 
+// One row of a row-major matrix as a buffer descriptor: row_bytes bytes at base + row*row_bytes
+// (row must be wave-uniform, so the address arithmetic runs on the scalar unit; any matrix
+// size).  A lane offset at or beyond row_bytes reads zeros, and a store there is dropped.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(const void *base, uint32_t row,
+                                                                 uint32_t row_bytes) {
+  const char *p = static_cast<const char *>(base) + static_cast<uint64_t>(row) * row_bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(p), 0, static_cast<int>(row_bytes), 0x00020000);
+}
+// N bytes (4, 8 or 16) per lane through a descriptor, as dwords
+template <int N>
+__device__ __forceinline__ vec_t<uint32_t, N / 4> descriptor_load(__amdgpu_buffer_rsrc_t r, uint32_t lane_bytes) {
+  static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 bytes per lane");
+  if constexpr (N == 4) {
+    vec_t<uint32_t, 1> v;
+    v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, lane_bytes, 0, 0);
+    return v;
+  } else if constexpr (N == 8) {
+    return __builtin_amdgcn_raw_buffer_load_b64(r, lane_bytes, 0, 0);
+  } else {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, lane_bytes, 0, 0);
+  }
+}
+template <int N>
+__device__ __forceinline__ void descriptor_store(__amdgpu_buffer_rsrc_t r, uint32_t lane_bytes,
+                                                 const vec_t<uint32_t, N / 4> &v) {
+  static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 bytes per lane");
+  if constexpr (N == 4) __builtin_amdgcn_raw_buffer_store_b32(v[0], r, lane_bytes, 0, 0);
+  else if constexpr (N == 8) __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_bytes, 0, 0);
+  else __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_bytes, 0, 0);
+}
+
 // acc + a.lo*b.lo + a.hi*b.hi on two packed bf16 pairs (one instruction on gfx950)
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
   typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));

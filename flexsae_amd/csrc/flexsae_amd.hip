@@ -317,8 +317,9 @@ void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int6
                          float *dvals, float *s_final, int d_pad, float *loss_partial, int *status_flag,
                          int64_t cols, int col0, int slice_w, hipStream_t st) {
   const int64_t n_items = s->B * (cols / 128);
-  hipLaunchKernelGGL((hier_train_kernel<WT, PT, KMAX>),
-                     dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
+  // K == KMAX (the usual powers of two) runs the variant without per-step bound tests
+  const auto kernel = s->K == KMAX ? hier_train_kernel<WT, PT, KMAX, true> : hier_train_kernel<WT, PT, KMAX, false>;
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
                      indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
                      coef, slot, P, dvals, s_final, d_pad, loss_partial, status_flag, n_items, s->B, col0,
                      slice_w, static_cast<int>(s->K), s->F, static_cast<int>(s->D));

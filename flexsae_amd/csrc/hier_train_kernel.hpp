@@ -47,9 +47,12 @@ struct RowPiece2<f16_t> {
 // i.e. sae_fwd_kernel and hier_sweep_kernel sharing one gather.  The gradient quantities are
 // those of a unit upstream gradient (c = 2/(B*K*D)); the caller scales them afterwards.
 // KMAX bounds K at compile time so that the row pieces can live in registers; steps k >= K
-// are skipped by uniform branches.  Every block of eight steps reduces its eight dvals dot
-// products with one transposed wave reduction.
-template <typename WT, typename PT, int KMAX>
+// are skipped by uniform branches, or not tested at all when FULL says K == KMAX.  Every block
+// of eight steps reduces its eight dvals dot products with one transposed wave reduction.
+// Row gathers and contribution stores go through per-row buffer descriptors: their address
+// arithmetic runs on the scalar unit, lanes beyond column D read zeros (so their dot products
+// vanish), and what such lanes store lands in the padding columns of P, which nobody reads.
+template <typename WT, typename PT, int KMAX, bool FULL>
 __global__ __launch_bounds__(256) void hier_train_kernel(
     const int64_t *__restrict__ indices, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
@@ -73,6 +76,13 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   const bool active = d0 < D;
   const int dsafe = active ? d0 : 0;
   const int64_t pair0 = b * K;
+  // Each phase tests k < K against its own copy of K: sharing the 128 comparison results
+  // between the phases costs more (scalar registers spilled into vector lanes) than redoing them.
+  auto k_bound = [&]() {
+    int kb = K;
+    asm volatile("" : "+s"(kb));
+    return kb;
+  };
 
   int my_row[KC], my_slot[KC];
   float my_val[KC], my_dval[KC];
@@ -98,12 +108,17 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
 
   // all gathers at once
   raw_t raw[KMAX];
-  const S_t *__restrict__ W = static_cast<const S_t *>(weight);
+  const uint32_t w_row_bytes = static_cast<uint32_t>(D) * sizeof(S_t);
+  const uint32_t w_lane_bytes = static_cast<uint32_t>(d0) * sizeof(S_t);  // beyond the row if !active
+  {
+    const int kb = k_bound();
 #pragma unroll
-  for (int k = 0; k < KMAX; ++k) {
-    if (k < K) {  // uniform
-      const int64_t row = bcast_i32(my_row[k / kWave], k % kWave);
-      raw[k] = *reinterpret_cast<const raw_t *>(W + row * D + dsafe);
+    for (int k = 0; k < KMAX; ++k) {
+      if (FULL || k < kb) {  // uniform
+        const uint32_t row = static_cast<uint32_t>(bcast_i32(my_row[k / kWave], k % kWave));
+        const auto dw = descriptor_load<sizeof(raw_t)>(row_descriptor(weight, row, w_row_bytes), w_lane_bytes);
+        __builtin_memcpy(&raw[k], &dw, sizeof(raw_t));
+      }
     }
   }
 
@@ -117,9 +132,10 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   }
 
   // forward walk
+  const int kb_fwd = k_bound();
 #pragma unroll
   for (int k = 0; k < KMAX; ++k) {
-    if (k < K) {  // uniform
+    if (FULL || k < kb_fwd) {  // uniform
       const float v = bcast_f32(my_val[k / kWave], k % kWave);
       float w[VEC];
       Piece::unpack(raw[k], w);
@@ -139,17 +155,20 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   float S[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; ++i) S[i] = 0.f;
+  const int kb_rev = k_bound();
+  const uint32_t p_row_bytes = static_cast<uint32_t>(slice_w) * sizeof(typename Traits<PT>::store_t);
+  const uint32_t p_lane_bytes = static_cast<uint32_t>(pc) * sizeof(typename Traits<PT>::store_t);
 #pragma unroll
   for (int k8 = KMAX - 8; k8 >= 0; k8 -= 8) {
-    if (k8 < K) {  // uniform
+    if (FULL || k8 < kb_rev) {  // uniform
       float dots[8];
 #pragma unroll
       for (int u = 7; u >= 0; --u) {
         const int k = k8 + u;
         dots[u] = 0.f;
-        if (k < K) {  // uniform
+        if (FULL || k < kb_rev) {  // uniform
           const float v = bcast_f32(my_val[k / kWave], k % kWave);
-          const int64_t prow = static_cast<uint32_t>(bcast_i32(my_slot[k / kWave], k % kWave));
+          const uint32_t prow = static_cast<uint32_t>(bcast_i32(my_slot[k / kWave], k % kWave));
           // Without this the compiler reuses the unpacked values of the forward walk, which
           // doubles the registers held across the two walks; re-unpacking costs one op per value.
           raw_t rk = raw[k];
@@ -164,8 +183,16 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
             dot = fmaf(w[i], S[i], dot);
             e[i] = fmaf(-w[i], v, e[i]);
           }
-          if (active) store_vec<PT, VEC>(P, prow * slice_w + pc, contrib);
-          dots[u] = active ? dot : 0.f;
+          vec_t<uint32_t, VEC * sizeof(typename Traits<PT>::store_t) / 4> packed;
+          if constexpr (Traits<PT>::dtype == FLEXSAE_BF16) {
+            packed[0] = f32x2_to_bf16x2_bits(contrib[0], contrib[1]);
+          } else {
+            static_assert(Traits<PT>::dtype == FLEXSAE_F32, "contributions are staged as bf16 or fp32");
+            packed[0] = __float_as_uint(contrib[0]);
+            packed[1] = __float_as_uint(contrib[1]);
+          }
+          descriptor_store<sizeof(packed)>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
+          dots[u] = dot;  // zero where the lane is beyond column D: its w is zero
         }
       }
       const float tot = wave_sum8_transposed(dots);  // lane L: total of step k8 + (L & 7)
