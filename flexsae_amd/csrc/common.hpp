@@ -276,13 +276,61 @@ __device__ __forceinline__ vec_t<uint32_t, N / 4> descriptor_load(__amdgpu_buffe
     return __builtin_amdgcn_raw_buffer_load_b128(r, lane_bytes, 0, 0);
   }
 }
-template <int N>
+// NT: non-temporal (streaming) store
+template <int N, bool NT = false>
 __device__ __forceinline__ void descriptor_store(__amdgpu_buffer_rsrc_t r, uint32_t lane_bytes,
                                                  const vec_t<uint32_t, N / 4> &v) {
   static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 bytes per lane");
-  if constexpr (N == 4) __builtin_amdgcn_raw_buffer_store_b32(v[0], r, lane_bytes, 0, 0);
-  else if constexpr (N == 8) __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_bytes, 0, 0);
-  else __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_bytes, 0, 0);
+  constexpr int kAux = NT ? 2 : 0;  // cache-policy bits of the instruction: bit 1 = nt
+  if constexpr (N == 4) __builtin_amdgcn_raw_buffer_store_b32(v[0], r, lane_bytes, 0, kAux);
+  else if constexpr (N == 8) __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_bytes, 0, kAux);
+  else __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_bytes, 0, kAux);
+}
+
+// VEC consecutive elements of row `row` (wave-uniform) of a row-major matrix, starting at column
+// d0, as stored.  Lanes with d0 beyond the row get zeros.  Pieces of at least four bytes go
+// through a row descriptor (address arithmetic on the scalar unit).
+template <typename T, int VEC>
+__device__ __forceinline__ raw_vec_t<T, VEC> gather_row_piece(const void *base, uint32_t row, int D, int d0) {
+  using S = typename Traits<T>::store_t;
+  constexpr int kBytes = VEC * static_cast<int>(sizeof(S));
+  raw_vec_t<T, VEC> out;
+  if constexpr (kBytes >= 4) {
+    const auto dw = descriptor_load<kBytes>(row_descriptor(base, row, static_cast<uint32_t>(D) * sizeof(S)),
+                                            static_cast<uint32_t>(d0) * sizeof(S));
+    __builtin_memcpy(&out, &dw, kBytes);
+  } else {
+    out = load_raw<T, VEC>(base, static_cast<int64_t>(row) * D + (d0 < D ? d0 : 0));
+    if (d0 >= D) out = raw_vec_t<T, VEC>{};
+  }
+  return out;
+}
+
+// x[0..VEC) rounded to T and stored at row `row` (wave-uniform), column `col`, of a row-major
+// matrix with `ld` columns; col + VEC <= ld must hold for every lane.  NT: streaming store.
+template <typename T, int VEC, bool NT>
+__device__ __forceinline__ void scatter_row_piece(void *base, uint32_t row, int ld, int col, const float (&x)[VEC]) {
+  using S = typename Traits<T>::store_t;
+  constexpr int kBytes = VEC * static_cast<int>(sizeof(S));
+  if constexpr (kBytes >= 4) {
+    vec_t<uint32_t, kBytes / 4> packed;
+    if constexpr (Traits<T>::dtype == FLEXSAE_BF16) {
+#pragma unroll
+      for (int i = 0; i < VEC / 2; ++i) packed[i] = f32x2_to_bf16x2_bits(x[2 * i], x[2 * i + 1]);
+    } else if constexpr (Traits<T>::dtype == FLEXSAE_F32) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) packed[i] = __float_as_uint(x[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC / 2; ++i)
+        packed[i] = static_cast<uint32_t>(f32_to_f16_bits(x[2 * i])) |
+                    (static_cast<uint32_t>(f32_to_f16_bits(x[2 * i + 1])) << 16);
+    }
+    descriptor_store<kBytes, NT>(row_descriptor(base, row, static_cast<uint32_t>(ld) * sizeof(S)),
+                                   static_cast<uint32_t>(col) * sizeof(S), packed);
+  } else {
+    store_vec<T, VEC, NT>(base, static_cast<int64_t>(row) * ld + col, x);
+  }
 }
 
 // acc + a.lo*b.lo + a.hi*b.hi on two packed bf16 pairs (one instruction on gfx950)

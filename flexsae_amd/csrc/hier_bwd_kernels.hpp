@@ -147,6 +147,8 @@ __global__ __launch_bounds__(256) void hier_sweep_kernel(
 #pragma unroll
   for (int i = 0; i < VEC; ++i) S[i] = 0.f;
 
+  constexpr int UB = U / 8;  // blocks of eight steps whose gathers are in flight together
+  static_assert(U % 8 == 0, "the prefetch depth counts blocks of eight steps");
   const int64_t pair0 = b * K;
   for (int k0 = ((K - 1) / kWave) * kWave; k0 >= 0; k0 -= kWave) {
     const int kk = k0 + lane;
@@ -167,39 +169,53 @@ __global__ __launch_bounds__(256) void hier_sweep_kernel(
     const int n = (K - k0) < kWave ? (K - k0) : kWave;  // uniform
     float my_dval = 0.f;
 
-    auto step = [&](int j, const float(&w)[VEC]) {
-      const float v = bcast_f32(my_val, j);
-      const int64_t prow = static_cast<uint32_t>(bcast_i32(my_slot, j));
-      float contrib[VEC];
-      float dot = 0.f;
+    // Steps run from n-1 down to 0 in aligned blocks of eight; the eight dot products of a block
+    // share one transposed wave reduction, whose result for step j lands in lane j.  Lanes beyond
+    // column D gather zeros, so their dot products vanish, and what they store lands in the
+    // padding columns of P, which nobody reads.
+    for (int m = ((n + 7) >> 3) - 1; m >= 0; m -= UB) {
+      raw_vec_t<WT, VEC> w[UB][8];
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) {
-        S[i] = fmaf(scale, e[i], S[i]);
-        contrib[i] = S[i] * v;
-        dot = fmaf(w[i], S[i], dot);
-        e[i] = fmaf(-w[i], v, e[i]);
-      }
-      if (active) store_vec<PT, VEC>(P, prow * slice_w + pc, contrib);
-      dot = wave_sum_bcast(active ? dot : 0.f);
-      if (lane == j) my_dval = dot;
-    };
-
-    int j = n - 1;
-    for (; j - (U - 1) >= 0; j -= U) {
-      float w[U][VEC];
+      for (int ub = 0; ub < UB; ++ub) {
+        if (m - ub >= 0) {  // uniform
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int64_t row = bcast_i32(my_row, j - u);
-        load_vec<WT, VEC>(weight, row * D + dsafe, w[u]);
+          for (int q = 0; q < 8; ++q) {
+            const int j = (m - ub) * 8 + q;
+            const int jj = j < n ? j : (n - 1);  // past the end: re-read the last row
+            w[ub][q] = gather_row_piece<WT, VEC>(weight, static_cast<uint32_t>(bcast_i32(my_row, jj)), D, d0);
+          }
+        }
       }
 #pragma unroll
-      for (int u = 0; u < U; ++u) step(j - u, w[u]);
-    }
-    for (; j >= 0; --j) {
-      float w[VEC];
-      const int64_t row = bcast_i32(my_row, j);
-      load_vec<WT, VEC>(weight, row * D + dsafe, w);
-      step(j, w);
+      for (int ub = 0; ub < UB; ++ub) {
+        if (m - ub >= 0) {  // uniform
+          float dots[8];
+#pragma unroll
+          for (int q = 7; q >= 0; --q) {
+            const int j = (m - ub) * 8 + q;
+            dots[q] = 0.f;
+            if (j < n) {  // uniform
+              const float v = bcast_f32(my_val, j);
+              const uint32_t prow = static_cast<uint32_t>(bcast_i32(my_slot, j));
+              float wj[VEC], contrib[VEC];
+              unpack_raw<WT, VEC>(w[ub][q], wj);
+              float dot = 0.f;
+#pragma unroll
+              for (int i = 0; i < VEC; ++i) {
+                S[i] = fmaf(scale, e[i], S[i]);
+                contrib[i] = S[i] * v;
+                dot = fmaf(wj[i], S[i], dot);
+                e[i] = fmaf(-wj[i], v, e[i]);
+              }
+              // no streaming hint: the slice is read back at once by the segment reduction
+              scatter_row_piece<PT, VEC, false>(P, prow, slice_w, pc, contrib);
+              dots[q] = dot;
+            }
+          }
+          const float tot = wave_sum8_transposed(dots);  // lane L: total of step 8*(m-ub) + (L & 7)
+          if ((lane >> 3) == (m - ub)) my_dval = tot;
+        }
+      }
     }
     if (kk < K) unsafeAtomicAdd(dvals + pair0 + kk, my_dval);
   }

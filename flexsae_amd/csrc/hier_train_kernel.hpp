@@ -3,6 +3,10 @@
 
 #include "common.hpp"
 
+#ifndef FLEXSAE_TRAIN_NT
+#define FLEXSAE_TRAIN_NT true
+#endif
+
 namespace flexsae {
 
 // A gathered piece of a weight row (two consecutive columns) kept in raw form.
@@ -191,7 +195,7 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
             packed[0] = __float_as_uint(contrib[0]);
             packed[1] = __float_as_uint(contrib[1]);
           }
-          descriptor_store<sizeof(packed)>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
+          descriptor_store<sizeof(packed), FLEXSAE_TRAIN_NT>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
           dots[u] = dot;  // zero where the lane is beyond column D: its w is zero
         }
       }

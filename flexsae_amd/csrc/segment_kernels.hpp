@@ -7,6 +7,10 @@
 
 #include "common.hpp"
 
+#ifndef FLEXSAE_REDUCE_NT
+#define FLEXSAE_REDUCE_NT true
+#endif
+
 namespace flexsae {
 
 constexpr int kSegChunk = 64;  // rows per chunk; groups longer than this count as "long"
@@ -14,7 +18,7 @@ constexpr int kSegChunk = 64;  // rows per chunk; groups longer than this count 
 // acc += sum of rows [r0, r0+n) of X (row stride `ld` elements) over the lane's VEC columns at pc.
 // Rows are fetched U at a time; a group that reaches past the end re-reads the last row (a cache
 // hit) instead of falling back to one load at a time, so short groups keep all loads in flight.
-template <typename PT, int VEC, int U>
+template <typename PT, int VEC, int U, bool NT = false>
 __device__ __forceinline__ void accumulate_rows(const void *__restrict__ X, int64_t r0, int n,
                                                 int64_t ld, int pc, float (&acc)[VEC]) {
   for (int j = 0; j < n; j += U) {
@@ -22,7 +26,7 @@ __device__ __forceinline__ void accumulate_rows(const void *__restrict__ X, int6
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int jj = (j + u) < n ? (j + u) : (n - 1);
-      load_vec<PT, VEC>(X, (r0 + jj) * ld + pc, x[u]);
+      unpack_raw<PT, VEC>(load_raw<PT, VEC, NT>(X, (r0 + jj) * ld + pc), x[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -86,13 +90,13 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
       float acc[VEC];
 #pragma unroll
       for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-      accumulate_rows<PT, VEC, U>(P, s0, static_cast<int>(n), slice_w, pc, acc);
+      accumulate_rows<PT, VEC, U, FLEXSAE_REDUCE_NT>(P, s0, static_cast<int>(n), slice_w, pc, acc);
       if (scale) {  // the rows were produced for a unit upstream gradient
         const float g = scale[0];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] *= g;
       }
-      if (d0 < D) store_vec<GT, VEC>(out, f * D + d0, acc);
+      if (d0 < D) store_vec<GT, VEC, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
     }
     return;
   }
@@ -109,7 +113,7 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-    accumulate_rows<PT, VEC, U>(P, c.s0, static_cast<int>(c.s1 - c.s0), slice_w, pc, acc);
+    accumulate_rows<PT, VEC, U, FLEXSAE_REDUCE_NT>(P, c.s0, static_cast<int>(c.s1 - c.s0), slice_w, pc, acc);
     store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
   }
 }
