@@ -170,11 +170,23 @@ __device__ __forceinline__ float wave_sum_bcast(float v) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// z(lane) + z(lane^16) + z(lane^32) + z(lane^48) in every lane, with the lane-swap instructions
+// of gfx950 (vector ALU only; a shuffle through the LDS crossbar would cost a round trip each).
+__device__ __forceinline__ float add_across_rows(float z) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  // swaps the odd 16-lane rows of the first operand with the even rows of the second
+  const u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(z), __float_as_uint(z), false, false);
+  z = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  // swaps the upper 32 lanes of the first operand with the lower 32 of the second
+  const u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(z), __float_as_uint(z), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Sum over the 64 lanes of eight values per lane at once: returns, in lane L, the wave-wide
 // total of d[L & 7].  Three exchange stages inside each group of 8 lanes halve the number of
 // live values while doubling the lanes summed (partner L^7, then L^2, then L^1: together they
 // generate the whole group), then three stages add the eight groups (L^8 by a row rotation,
-// L^16 and L^32 by lane permutes).  About 3.5 VALU operations per value instead of 12.
+// L^16 and L^32 by lane swaps).  About 3.5 VALU operations per value instead of 12.
 __device__ __forceinline__ float wave_sum8_transposed(const float (&d)[8]) {
   const int lane = lane_id();
   const bool b2 = (lane & 4) != 0, b1 = (lane & 2) != 0, b0 = (lane & 1) != 0;
@@ -196,8 +208,7 @@ __device__ __forceinline__ float wave_sum8_transposed(const float (&d)[8]) {
   const float give = b0 ? q[0] : q[1];
   float z = keep + dpp_move<0xB1>(give);  // quad_perm [1,0,3,2]: lane ^ 1
   z += dpp_move<0x128>(z);                // row_ror:8 within the 16-lane row: lane ^ 8
-  z += __shfl_xor(z, 16, kWave);
-  z += __shfl_xor(z, 32, kWave);
+  z = add_across_rows(z);
   return z;
 }
 

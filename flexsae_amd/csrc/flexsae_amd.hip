@@ -511,12 +511,12 @@ void launch_topk_slices(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t s
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
-    const int64_t n_short_blocks = ceil_div(s->F * tps, static_cast<int64_t>(kWavesPerBlock));
+    const int64_t n_short_blocks = ceil_div(s->F, static_cast<int64_t>(kWavesPerBlock));
     const size_t resid_bytes =
         static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * sizeof(typename Traits<RT>::store_t);
     hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, RT, VEC, FLEXSAE_TOPK_U>),
-                       dim3(kLongBlocks + static_cast<unsigned>(n_short_blocks)), dim3(kBlock), 0, st, begin, map,
-                       long_count, long_list, chunk_begin,
+                       dim3(kLongBlocks + static_cast<unsigned>(n_short_blocks), static_cast<unsigned>(tps)),
+                       dim3(kBlock), 0, st, begin, map, long_count, long_list, chunk_begin,
                        reinterpret_cast<const vec_t<uint32_t, 2> *>(ws + pl.off_slotbv), weight, vals,
                        s->vals_dtype, resid, grad_out, coef, dW, dv_part, n_pairs, partial, kLongBlocks, tps,
                        static_cast<int>(col0), sw, s->F, K, D, static_cast<uint32_t>(resid_bytes));

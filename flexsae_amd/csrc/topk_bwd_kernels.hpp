@@ -74,11 +74,13 @@ __device__ __forceinline__ void topk_accumulate_slots(
   }
 }
 
-// One short latent (at most kSegChunk pairs) for one tile: the pair records of the latent are one
+// One short latent (1 to kSegChunk pairs) for one tile: the pair records of the latent are one
 // contiguous load, the residual rows are gathered through a buffer descriptor (no vector ALU work
 // for addresses) eight at a time with the next eight already requested, and each group of
-// eight shares one transposed wave reduction for the dvals dot products.  With bf16 weights and
-// a bf16 residual copy the products run on packed pairs (dot2) without unpacking.
+// eight shares one transposed wave reduction for the dvals dot products.  Groups are always
+// processed in full: slots past the end re-read the last row (a cache hit) with a val of zero,
+// which keeps the inner code free of branches.  With bf16 weights and a bf16 residual copy the
+// products run on packed pairs (dot2) without unpacking.
 template <typename WT, typename GT, typename RT, int VEC>
 __device__ __forceinline__ void topk_short_latent(
     const vec_t<uint32_t, 2> *__restrict__ slot_bv, const void *__restrict__ weight, int vals_dtype,
@@ -92,6 +94,7 @@ __device__ __forceinline__ void topk_short_latent(
   const bool late_scale = kDot2 && vals_dtype == FLEXSAE_BF16;  // vals enter the dot2 as they are
 
   const raw_vec_t<WT, VEC> wraw = load_raw<WT, VEC, FLEXSAE_TOPK_NT>(weight, f * D + (active ? d0 : 0));
+  // lanes past the end hold row 0 and a val of zero
   const vec_t<uint32_t, 2> bv = lane < n ? __builtin_nontemporal_load(slot_bv + b0 + lane) : vec_t<uint32_t, 2>{0u, 0u};
   const int my_b = static_cast<int>(bv[0]);
   const uint32_t vbits = bv[1];
@@ -99,17 +102,12 @@ __device__ __forceinline__ void topk_short_latent(
   raw_vec_t<RT, VEC> buf_a[8], buf_b[8];
   auto issue = [&](raw_vec_t<RT, VEC>(&buf)[8], int j) {
 #pragma unroll
-    for (int u = 0; u < 8; u += 4) {
-      if (j + u < n) {  // uniform
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int jj = (j + u + q) < n ? (j + u + q) : (n - 1);  // past the end: re-read the last row
-          buf[u + q] = gather_raw<RT, VEC>(rows_src, lane_off, static_cast<uint32_t>(bcast_i32(my_b, jj)) * row_stride);
-        }
-      }
+    for (int u = 0; u < 8; ++u) {
+      const int jj = (j + u) < n ? (j + u) : (n - 1);
+      buf[u] = gather_raw<RT, VEC>(rows_src, lane_off, static_cast<uint32_t>(bcast_i32(my_b, jj)) * row_stride);
     }
   };
-  if (n > 0) issue(buf_a, 0);
+  issue(buf_a, 0);
   if (n > 8) issue(buf_b, 8);
 
   float w[VEC], acc[VEC];
@@ -126,48 +124,45 @@ __device__ __forceinline__ void topk_short_latent(
     for (int i = 0; i < VEC / 2; ++i)
       if (!active) ww[i] = 0u;
   }
-  const float v = __uint_as_float(vbits) * (late_scale ? 1.f : scale);  // lanes >= n are never read
+  const float v = __uint_as_float(vbits) * (late_scale ? 1.f : scale);
   float my_dot = 0.f;
   auto consume = [&](const raw_vec_t<RT, VEC>(&rows)[8], int j) {  // slots j .. j+7 of the latent
     float dots[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      dots[u] = 0.f;
-      if (j + u < n) {  // uniform
-        float dot = 0.f;
-        if constexpr (kDot2) {
-          uint32_t xw[VEC / 2];
-          __builtin_memcpy(xw, &rows[u], sizeof(xw));
+      float dot = 0.f;
+      if constexpr (kDot2) {
+        uint32_t xw[VEC / 2];
+        __builtin_memcpy(xw, &rows[u], sizeof(xw));
 #pragma unroll
-          for (int i = 0; i < VEC / 2; ++i) dot = dot2_bf16(xw[i], ww[i], dot);
-          if (late_scale) {  // uniform
-            // a bf16 val widened to fp32 keeps its 16 bits in the upper half
-            const uint32_t v_hi = static_cast<uint32_t>(bcast_i32(static_cast<int>(vbits), j + u));
-            const uint32_t v_lo = v_hi >> 16;
+        for (int i = 0; i < VEC / 2; ++i) dot = dot2_bf16(xw[i], ww[i], dot);
+        if (late_scale) {  // uniform
+          // a bf16 val widened to fp32 keeps its 16 bits in the upper half
+          const uint32_t v_hi = static_cast<uint32_t>(bcast_i32(static_cast<int>(vbits), j + u));
+          const uint32_t v_lo = v_hi >> 16;
 #pragma unroll
-            for (int i = 0; i < VEC / 2; ++i) {
-              acc[2 * i] = dot2_bf16(xw[i], v_lo, acc[2 * i]);
-              acc[2 * i + 1] = dot2_bf16(xw[i], v_hi, acc[2 * i + 1]);
-            }
-          } else {
-            float x[VEC];
-            unpack_raw<RT, VEC>(rows[u], x);
-            const float vj = bcast_f32(v, j + u);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] = fmaf(vj, x[i], acc[i]);
+          for (int i = 0; i < VEC / 2; ++i) {
+            acc[2 * i] = dot2_bf16(xw[i], v_lo, acc[2 * i]);
+            acc[2 * i + 1] = dot2_bf16(xw[i], v_hi, acc[2 * i + 1]);
           }
         } else {
           float x[VEC];
           unpack_raw<RT, VEC>(rows[u], x);
           const float vj = bcast_f32(v, j + u);
 #pragma unroll
-          for (int i = 0; i < VEC; ++i) {
-            acc[i] = fmaf(vj, x[i], acc[i]);
-            dot = fmaf(x[i], w[i], dot);
-          }
+          for (int i = 0; i < VEC; ++i) acc[i] = fmaf(vj, x[i], acc[i]);
         }
-        dots[u] = dot;
+      } else {
+        float x[VEC];
+        unpack_raw<RT, VEC>(rows[u], x);
+        const float vj = bcast_f32(v, j + u);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          acc[i] = fmaf(vj, x[i], acc[i]);
+          dot = fmaf(x[i], w[i], dot);
+        }
       }
+      dots[u] = dot;
     }
     const float tot = wave_sum8_transposed(dots);  // lane L: total of slot j + (L & 7)
     if ((lane >> 3) == (j >> 3)) my_dot = tot;
@@ -192,9 +187,9 @@ __device__ __forceinline__ void topk_short_latent(
 // Blocks [0, n_long_blocks): long latents, one wavefront per (64-pair chunk, tile): stores its
 // dvals shares, leaves its dW contribution in partial[chunk, slice column] (fp32) for
 // seg_reduce_long_finalize_kernel (next launch).  They come first so hot latents start at once.
-// Remaining blocks: one wavefront per (tile of the slice, latent f), tile-major, so that at any
-// moment the waves in flight share one B x tile slice of resid (L2-sized); see
-// topk_short_latent.  tile = 64*VEC columns, lane l owning VEC consecutive columns.
+// Remaining blocks: one wavefront per (tile of the slice = blockIdx.y, latent f); blocks are
+// handed out x first, i.e. tile-major, so that at any moment the waves in flight share one
+// B x tile slice of resid (L2-sized); see topk_short_latent.  tile = 64*VEC columns, lane l owning VEC consecutive columns.
 // dW[f, tile] is written exactly once, in the gradient's final dtype; latents without pairs
 // get zeros.
 template <typename WT, typename GT, typename RT, int VEC, int U>
@@ -210,28 +205,33 @@ __global__ __launch_bounds__(256) void topk_bwd_kernel(
   const int lane = lane_id();
   const float scale = coef * grad_out[0];
   if (blockIdx.x >= n_long_blocks) {
-    const int64_t item =
-        static_cast<int64_t>(blockIdx.x - n_long_blocks) * (blockDim.x >> 6) + wave_in_block();
-    if (item >= F * tps) return;  // uniform per wavefront
-    const int t = static_cast<int>(item / F);
-    const int64_t f = item - static_cast<int64_t>(t) * F;
+    // blockIdx.y = tile of the slice, blockIdx.x - n_long_blocks = group of latents
+    const int64_t f = static_cast<int64_t>(blockIdx.x - n_long_blocks) * (blockDim.x >> 6) + wave_in_block();
+    if (f >= F) return;  // uniform per wavefront
+    const int t = static_cast<int>(blockIdx.y);
     const uint32_t b0 = begin[f];
     const uint32_t n = begin[f + 1] - b0;
     if (n > static_cast<uint32_t>(kSegChunk)) return;  // chunk role
+    const int d0 = col0 + t * (kWave * VEC) + lane * VEC;
+    if (n == 0) {  // unused latent: zeros
+      const float zero[VEC] = {};
+      if (d0 < D) store_vec<GT, VEC, FLEXSAE_TOPK_NT>(dW, f * D + d0, zero);
+      return;
+    }
     const GatherSource rows_src = make_gather_source(resid, resid_bytes);
     topk_short_latent<WT, GT, RT, VEC>(
         slot_bv, weight, vals_dtype, rows_src, static_cast<uint32_t>(D) * sizeof(typename Traits<RT>::store_t), scale,
-        dW, dv_part + (col0 / (kWave * VEC) + t) * n_pairs, f, b0, static_cast<int>(n),
-        col0 + t * (kWave * VEC) + lane * VEC, D);
+        dW, dv_part + (col0 / (kWave * VEC) + t) * n_pairs, f, b0, static_cast<int>(n), d0, D);
     return;
   }
   const uint32_t n_long = *long_count;
   if (n_long == 0) return;
   const uint32_t n_chunks = chunk_begin[n_long];
   const int64_t total = static_cast<int64_t>(n_chunks) * tps;
-  const int64_t n_waves = static_cast<int64_t>(n_long_blocks) * (blockDim.x >> 6);
-  for (int64_t wk = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); wk < total;
-       wk += n_waves) {
+  const int64_t n_waves = static_cast<int64_t>(n_long_blocks) * gridDim.y * (blockDim.x >> 6);
+  for (int64_t wk = (static_cast<int64_t>(blockIdx.y) * n_long_blocks + blockIdx.x) * (blockDim.x >> 6) +
+                    wave_in_block();
+       wk < total; wk += n_waves) {
     // tile-major over the work list as well
     const int t = static_cast<int>(wk / n_chunks);
     const uint32_t chunk = static_cast<uint32_t>(wk - static_cast<int64_t>(t) * n_chunks);
