@@ -262,7 +262,7 @@ struct HierBwdPlan {
   size_t n_pairs;          // B * K
   size_t n_rows;           // B
   size_t n_partial_rows;   // upper bound on the number of 64-pair chunks of long latents
-  size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_sfinal, off_colsum, off_loss, off_partial;  // per-slice buffers follow
+  size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_sfinal, off_colsum, off_loss, off_dvpart, off_partial;  // per-slice buffers follow
   size_t n_loss_partials;  // training-step kernel: one per (128-column tile, row)
   size_t fixed_bytes;      // everything that does not depend on the slice width
 };
@@ -294,6 +294,10 @@ HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
   p.off_loss = off;
   p.n_loss_partials = p.n_rows * static_cast<size_t>(p.d_pad / 128 + 1);
   off += round_up(p.n_loss_partials * 4, kAlign);
+  // per-tile shares of dvals, [number of tiles, B*K] fp32, added up in tile order afterwards
+  // (tiles are 128 columns in the training-step kernel, 64*vec in the sweep kernel)
+  p.off_dvpart = off;
+  off += round_up(static_cast<size_t>(p.d_pad / (p.tile < 128 ? p.tile : 128)) * p.n_pairs * 4, kAlign);
   p.off_partial = off;
   p.fixed_bytes = off;
   return p;
@@ -372,6 +376,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
   void *P = ws + pl.off_partial + hier_partial_bytes(pl, slice_w);
   float *s_final = reinterpret_cast<float *>(ws + pl.off_sfinal);
+  float *dv_part = reinterpret_cast<float *>(ws + pl.off_dvpart);
   float *colsum_part = reinterpret_cast<float *>(ws + pl.off_colsum);
   const int n_chunks = static_cast<int>(ceil_div(s->B, kColsumRows));
   const int d_pad = static_cast<int>(pl.d_pad);
@@ -382,13 +387,13 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     const int tps = static_cast<int>(cols / pl.tile);
     const int64_t sweep_items = s->B * tps;
     if (train && do_sweep) {
-      launch_train_kernel_k<WT, PT>(s, *train, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,
+      launch_train_kernel_k<WT, PT>(s, *train, indices, weight, vals, coef, slot, P, dv_part, s_final, d_pad,
                                     reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
                                     static_cast<int>(col0), sw, st);
     } else if (do_sweep)
       hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, FLEXSAE_SWEEP_U>),
                          dim3(static_cast<unsigned>(ceil_div(sweep_items, kWavesPerBlock))), dim3(kBlock),
-                         0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dvals,
+                         0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dv_part,
                          s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F,
                          D);
     if (!do_reduce) continue;
@@ -402,6 +407,9 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
+  // dvals = its per-tile shares added in tile order
+  hipLaunchKernelGGL(hier_dvals_finalize_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, dv_part,
+                     static_cast<int>(pl.d_pad / (train ? 128 : pl.tile)), s->B * s->K, dvals);
   // dbias = column sums of s_final over the rows, in a fixed order
   hipLaunchKernelGGL(colsum_partial_kernel,
                      dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
@@ -693,7 +701,6 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
     return FLEXSAE_ERR_ALIGNMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint8_t *ws = static_cast<uint8_t *>(workspace);
-  if (!(flags & (FLEXSAE_BWD_OUTPUTS_PREZEROED | FLEXSAE_BWD_REDUCE_ONLY))) zero_f32(dvals, s->B * s->K, st);
   uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
@@ -749,7 +756,6 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   if (defer_reduce && slice_w < pl.d_pad) return FLEXSAE_ERR_WORKSPACE;  // contributions must all fit
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint8_t *ws = static_cast<uint8_t *>(workspace);
-  if (!(flags & FLEXSAE_BWD_OUTPUTS_PREZEROED)) zero_f32(dvals, s->B * s->K, st);
   uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);

@@ -116,8 +116,8 @@ namespace flexsae {
 // position in the latent-major pair list, so that all rows of one latent are adjacent and a
 // segment reduction (segment_kernels.hpp) can stream them.  Only the columns
 // [col0, col0 + tps*64*VEC) of the problem (one "slice") are handled per launch, so P needs
-// B*K*slice_width elements.  dvals partial dot products are added across tiles with atomics
-// (one address per pair and tile: no contention).
+// B*K*slice_width elements.  Every tile leaves its share of the dvals dot products in dv_part;
+// hier_dvals_finalize_kernel adds the shares in tile order (deterministic).
 //
 // One wavefront per (tile of the slice, row b), tile-major: the wavefronts in flight at any
 // moment gather from the same 64*VEC-column slice of W, which is small enough to stay in the
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void hier_sweep_kernel(
     const int64_t *__restrict__ indices, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const float *__restrict__ resid,
     const float *__restrict__ grad_out, float coef, const uint32_t *__restrict__ slot,
-    void *__restrict__ P, float *__restrict__ dvals, float *__restrict__ s_final, int s_final_ld,
+    void *__restrict__ P, float *__restrict__ dv_part, float *__restrict__ s_final, int s_final_ld,
     int *status_flag, int64_t n_items, int64_t B, int col0, int slice_w, int K, int64_t F,
     int D) {
   const int lane = lane_id();
@@ -217,7 +217,8 @@ __global__ __launch_bounds__(256) void hier_sweep_kernel(
         }
       }
     }
-    if (kk < K) unsafeAtomicAdd(dvals + pair0 + kk, my_dval);
+    // this tile's share of dvals; hier_dvals_finalize_kernel adds the tiles up in order
+    if (kk < K) dv_part[(static_cast<int64_t>(col0 / (kWave * VEC)) + t) * (B * K) + pair0 + kk] = my_dval;
   }
   // the row's total S_{b,0} (its share of dbias) goes to s_final[b, column]; a column sum over
   // b follows (thousands of atomics per dbias element would serialise instead)
@@ -226,6 +227,17 @@ __global__ __launch_bounds__(256) void hier_sweep_kernel(
     for (int i = 0; i < VEC; ++i) S[i] = 0.f;
   }
   store_vec<float, VEC>(s_final, b * s_final_ld + col0 + pc, S);
+}
+
+// dvals[p] = sum over the column tiles of dv_part[tile, p], in tile order (deterministic).
+__global__ void hier_dvals_finalize_kernel(const float *__restrict__ dv_part, int n_tiles, int64_t n_pairs,
+                                           float *__restrict__ dvals) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < n_pairs; p += stride) {
+    float acc = 0.f;
+    for (int t = 0; t < n_tiles; ++t) acc += dv_part[t * n_pairs + p];
+    dvals[p] = acc;
+  }
 }
 
 }  // namespace flexsae

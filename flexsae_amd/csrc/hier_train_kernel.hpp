@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     const int64_t *__restrict__ indices, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
     const void *__restrict__ target, int target_dtype, float coef,
-    const uint32_t *__restrict__ slot, void *__restrict__ P, float *__restrict__ dvals,
+    const uint32_t *__restrict__ slot, void *__restrict__ P, float *__restrict__ dv_part,
     float *__restrict__ s_final, int s_final_ld, float *__restrict__ loss_partial,
     int *status_flag, int64_t n_items, int64_t B, int col0, int slice_w, int K, int64_t F, int D) {
   using Piece = RowPiece2<WT>;
@@ -206,7 +206,8 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
 #pragma unroll
   for (int c = 0; c < KC; ++c) {
     const int kk = c * kWave + lane;
-    if (kk < K) unsafeAtomicAdd(dvals + pair0 + kk, my_dval[c]);
+    // this tile's share of dvals; hier_dvals_finalize_kernel adds the tiles up in order
+    if (kk < K) dv_part[(static_cast<int64_t>(col0 / (kWave * VEC)) + t) * (B * K) + pair0 + kk] = my_dval[c];
   }
   if (!active) {
 #pragma unroll
