@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes.
+"""The five benchmark configurations at their full sizes.
 
 Configurations 1-3 are compared element by element with the CPU oracle (double accumulation).
 Configurations 4 and 5 are too large for that in a test's time budget, so they are checked

@@ -331,7 +331,7 @@ def test_topk_slice_width_does_not_change_the_result(shape, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_skewed_latents(mode, dtype):
     """Zipf-distributed per-row-unique indices with vals sorted descending (the shape of the
-    skewed BASELINE configuration, scaled down): a few latents appear in almost every row."""
+    skewed benchmark configuration, scaled down): a few latents appear in almost every row."""
     B, K, F, D = 512, 16, 4096, 512
     _announce("zipf", mode, dtype)
     args = make_inputs(B, K, F, D, dtype=dtype, seed=77, zipf_s=1.1, sort_vals=True, w_std=0.02)
