@@ -26,6 +26,9 @@ using namespace flexsae;
 #ifndef FLEXSAE_TOPK_U
 #define FLEXSAE_TOPK_U 4
 #endif
+#ifndef FLEXSAE_TOPK_VEC8
+#define FLEXSAE_TOPK_VEC8 1
+#endif
 #ifndef FLEXSAE_TOPK_RESID16
 #define FLEXSAE_TOPK_RESID16 1
 #endif
@@ -472,7 +475,12 @@ struct TopkBwdPlan {
 
 TopkBwdPlan plan_topk_bwd(const flexsae_shape *s) {
   TopkBwdPlan p;
+  // The reference hands its backward the residual gradient in the weight dtype
+  // (topk_kernels.py:52,221); for bf16 weights the gathers here read a bf16 copy as well.
+  p.resid16 = FLEXSAE_TOPK_RESID16 && s->weight_dtype == FLEXSAE_BF16;
   p.vec = (s->D % 4 == 0) ? 4 : (s->D % 2 == 0) ? 2 : 1;
+  // all-bf16: 16 bytes per lane (512-column tiles) halve the per-tile overheads
+  if (FLEXSAE_TOPK_VEC8 && p.resid16 && s->D % 8 == 0) p.vec = 8;
   p.tile = kWave * p.vec;
   p.d_pad = ceil_div(s->D, p.tile) * p.tile;
   p.n_pairs = static_cast<size_t>(s->B) * static_cast<size_t>(s->K);
@@ -486,9 +494,6 @@ TopkBwdPlan plan_topk_bwd(const flexsae_shape *s) {
   off += round_up((p.n_pairs / 65 + 1) * 4, kAlign);
   p.off_chunk = off;
   off += round_up((p.n_pairs / 65 + 2) * 4, kAlign);
-  // The reference hands its backward the residual gradient in the weight dtype
-  // (topk_kernels.py:52,221); for bf16 weights the gathers here read a bf16 copy as well.
-  p.resid16 = FLEXSAE_TOPK_RESID16 && s->weight_dtype == FLEXSAE_BF16;
   p.off_resid16 = off;
   if (p.resid16) off += round_up(static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * 2, kAlign);
   p.off_dvpart = off;  // per-tile shares of dvals: [d_pad / tile, B*K] fp32
@@ -874,7 +879,10 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
                        st, r16, resid, n);
     gather_src = r16;
   }
-  if (pl.vec == 4) {
+  if (pl.vec == 8) {
+    launch_topk_slices_g<bf16_t, bf16_t, 8>(s, pl, slice_w, begin, map, weight, vals, gather_src, grad_out, coef,
+                                            dW, dW_dtype, dvals, ws, st);
+  } else if (pl.vec == 4) {
     launch_topk_slices_w<4>(s, pl, slice_w, begin, map, weight, vals, gather_src, grad_out, coef, dW,
                             dW_dtype, dvals, ws, st);
   } else if (pl.vec == 2) {
