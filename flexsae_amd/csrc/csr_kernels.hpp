@@ -7,7 +7,8 @@
 namespace flexsae {
 
 // ---------------------------------------------------------------------------------
-// Pair list.  count -> exclusive scan -> fill -> sort each group ascending.
+// Pair list.  count (keeping each pair's rank in its group) -> exclusive scan -> fill -> sort
+// each group ascending.
 // ---------------------------------------------------------------------------------
 
 __global__ void fill_u32_kernel(uint32_t *__restrict__ p, int64_t n, uint32_t value) {
@@ -16,9 +17,12 @@ __global__ void fill_u32_kernel(uint32_t *__restrict__ p, int64_t n, uint32_t va
     p[i] = value;
 }
 
-// counts[f] += 1 for every pair; out-of-range indices are flagged and counted as latent 0.
+// counts[f] += 1 for every pair, and rank[p] = the value the counter had before: a position
+// inside the latent's group that is unique but depends on the order the atomics were served in
+// (the groups are sorted afterwards).  Out-of-range indices are flagged and counted as latent 0.
 __global__ void csr_count_kernel(const int64_t *__restrict__ indices, int64_t n_pairs, int64_t F,
-                                 uint32_t *__restrict__ counts, int *status_flag) {
+                                 uint32_t *__restrict__ counts, uint32_t *__restrict__ rank,
+                                 int *status_flag) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < n_pairs;
        p += stride) {
@@ -27,14 +31,14 @@ __global__ void csr_count_kernel(const int64_t *__restrict__ indices, int64_t n_
       if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
       f = 0;
     }
-    atomicAdd(counts + f, 1u);
+    rank[p] = atomicAdd(counts + f, 1u);
   }
 }
 
 // Exclusive scan of the per-latent counts in two launches.  Every block owns kScanBlockElems
 // consecutive latents: csr_scan_sums_kernel writes the block totals, csr_scan_apply_kernel
 // adds up the totals of the blocks before it (a few hundred values at most), scans its own
-// elements and writes begin[] and a copy for the fill cursor; the last block writes begin[F].
+// elements and writes begin[]; the last block writes begin[F].
 constexpr int kScanThreads = 256;
 constexpr int kScanPerThread = 8;
 constexpr int kScanBlockElems = kScanThreads * kScanPerThread;
@@ -65,7 +69,6 @@ __global__ __launch_bounds__(kScanThreads) void csr_scan_sums_kernel(const uint3
 }
 
 __global__ __launch_bounds__(kScanThreads) void csr_scan_apply_kernel(uint32_t *__restrict__ begin,
-                                                                      uint32_t *__restrict__ cursor,
                                                                       int64_t F,
                                                                       const uint32_t *__restrict__ block_sums) {
   __shared__ uint32_t smem[kScanThreads / kWave];
@@ -98,29 +101,27 @@ __global__ __launch_bounds__(kScanThreads) void csr_scan_apply_kernel(uint32_t *
   uint32_t run = block_off + wave_off + (inc - tsum);
 #pragma unroll
   for (int i = 0; i < kScanPerThread; ++i) {
-    if (i0 + i < F) {
-      begin[i0 + i] = run;
-      cursor[i0 + i] = run;
-    }
+    if (i0 + i < F) begin[i0 + i] = run;
     run += x[i];
   }
   if (blockIdx.x == gridDim.x - 1 && tid == kScanThreads - 1) begin[F] = run;
 }
 
+// map[begin[f] + rank[p]] = p: every pair goes to its group without any further atomic.
 __global__ void csr_fill_kernel(const int64_t *__restrict__ indices, int64_t n_pairs, int64_t F,
-                                uint32_t *__restrict__ cursor, uint32_t *__restrict__ map) {
+                                const uint32_t *__restrict__ begin, const uint32_t *__restrict__ rank,
+                                uint32_t *__restrict__ map) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < n_pairs;
        p += stride) {
     int64_t f = indices[p];
     if (static_cast<uint64_t>(f) >= static_cast<uint64_t>(F)) f = 0;
-    const uint32_t pos = atomicAdd(cursor + f, 1u);
-    map[pos] = static_cast<uint32_t>(p);
+    map[begin[f] + rank[p]] = static_cast<uint32_t>(p);
   }
 }
 
 // Sort every group ascending so that the list does not depend on the order in which the
-// fill kernel's atomics happened to be served.  One wavefront per latent: groups of up to
+// count kernel's atomics happened to be served.  One wavefront per latent: groups of up to
 // 64 pairs are rank-sorted in registers (pair ids are distinct); longer ones are appended
 // to long_list for csr_sort_long_kernel.
 __global__ __launch_bounds__(256) void csr_sort_short_kernel(const uint32_t *__restrict__ begin,

@@ -210,7 +210,7 @@ void zero_f32(float *p, int64_t n, hipStream_t st) {
 // cursor[F] | scan block sums[ceil(F/kScanBlockElems)] | long_count (one aligned slot) |
 // long_list[B*K/65 + 1]
 struct CsrScratch {
-  uint32_t *cursor;
+  uint32_t *rank;
   uint32_t *block_sums;
   uint32_t *long_count;
   uint32_t *long_list;
@@ -220,11 +220,11 @@ size_t csr_scan_sums_bytes(int64_t F) {
   return round_up(static_cast<size_t>(ceil_div(F, kScanBlockElems)) * 4, kAlign);
 }
 
-CsrScratch carve_csr_scratch(void *workspace, int64_t F) {
+CsrScratch carve_csr_scratch(void *workspace, int64_t F, int64_t n_pairs) {
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   CsrScratch sc;
-  sc.cursor = reinterpret_cast<uint32_t *>(ws);
-  ws += round_up(static_cast<size_t>(F) * 4, kAlign);
+  sc.rank = reinterpret_cast<uint32_t *>(ws);
+  ws += round_up(static_cast<size_t>(n_pairs) * 4, kAlign);
   sc.block_sums = reinterpret_cast<uint32_t *>(ws);
   ws += csr_scan_sums_bytes(F);
   sc.long_count = reinterpret_cast<uint32_t *>(ws);
@@ -240,14 +240,14 @@ void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
   hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, sc.long_count,
                      static_cast<int64_t>(1), 0u);
   hipLaunchKernelGGL(csr_count_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st,
-                     indices, n_pairs, F, begin, status_flag);
+                     indices, n_pairs, F, begin, sc.rank, status_flag);
   const unsigned scan_blocks = static_cast<unsigned>(ceil_div(F, kScanBlockElems));
   hipLaunchKernelGGL(csr_scan_sums_kernel, dim3(scan_blocks), dim3(kScanThreads), 0, st, begin, F,
                      sc.block_sums);
-  hipLaunchKernelGGL(csr_scan_apply_kernel, dim3(scan_blocks), dim3(kScanThreads), 0, st, begin,
-                     sc.cursor, F, sc.block_sums);
+  hipLaunchKernelGGL(csr_scan_apply_kernel, dim3(scan_blocks), dim3(kScanThreads), 0, st, begin, F,
+                     sc.block_sums);
   hipLaunchKernelGGL(csr_fill_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, indices,
-                     n_pairs, F, sc.cursor, map);
+                     n_pairs, F, begin, sc.rank, map);
   hipLaunchKernelGGL(csr_sort_short_kernel,
                      dim3(static_cast<unsigned>(ceil_div(F, kWavesPerBlock))), dim3(kBlock), 0, st,
                      begin, map, F, sc.long_count, sc.long_list);
@@ -374,7 +374,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const float *dw_scale = (flags & FLEXSAE_BWD_SCALE_BY_GRAD_OUT) ? grad_out : nullptr;
   const uint32_t *begin = reinterpret_cast<const uint32_t *>(ws + pl.off_begin);
   const uint32_t *slot = reinterpret_cast<const uint32_t *>(ws + pl.off_slot);
-  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
   uint32_t *chunk_begin = reinterpret_cast<uint32_t *>(ws + pl.off_chunk);
   float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
   void *P = ws + pl.off_partial + hier_partial_bytes(pl, slice_w);
@@ -708,7 +708,7 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
-  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
     csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
     hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
@@ -763,7 +763,7 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   uint32_t *begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
-  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F);
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
     csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
     hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
@@ -807,8 +807,8 @@ int flexsae_scale(void *dst, const void *src, int dtype, int64_t n, const float 
 
 size_t flexsae_csr_workspace_bytes(int64_t B, int64_t K, int64_t F) {
   if (B <= 0 || K <= 0 || F <= 0) return 0;
-  // cursor[F] | scan block sums | long_count (padded) | long_list[B*K/65 + 1]
-  return round_up(static_cast<size_t>(F) * 4, kAlign) + csr_scan_sums_bytes(F) + kAlign +
+  // rank[B*K] | scan block sums | long_count (padded) | long_list[B*K/65 + 1]
+  return round_up(static_cast<size_t>(B) * static_cast<size_t>(K) * 4, kAlign) + csr_scan_sums_bytes(F) + kAlign +
          round_up((static_cast<size_t>(B) * static_cast<size_t>(K) / 65 + 1) * 4, kAlign);
 }
 
@@ -821,7 +821,7 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
   if (!workspace || workspace_bytes < flexsae_csr_workspace_bytes(B, K, F) ||
       !aligned(workspace, kAlign))
     return FLEXSAE_ERR_WORKSPACE;
-  const CsrScratch sc = carve_csr_scratch(workspace, F);
+  const CsrScratch sc = carve_csr_scratch(workspace, F, B * K);
   csr_build_launch(indices, B, K, F, begin, map, sc, status_flag, static_cast<hipStream_t>(stream));
   return launch_status();
 }
