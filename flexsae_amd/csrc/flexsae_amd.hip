@@ -51,7 +51,8 @@ int check_shape(const flexsae_shape *s) {
   if (!valid_dtype(s->weight_dtype) || !valid_dtype(s->vals_dtype) || !valid_dtype(s->bias_dtype) ||
       !valid_dtype(s->target_dtype))
     return FLEXSAE_ERR_INVALID_ARGUMENT;
-  if (s->F >= (1LL << 31) || s->D >= (1LL << 31) || s->K >= (1LL << 31)) return FLEXSAE_ERR_UNSUPPORTED;
+  // D < 2^29: a row of any matrix here (at most 4 bytes per element) fits a buffer descriptor
+  if (s->F >= (1LL << 31) || s->D >= (1LL << 29) || s->K >= (1LL << 31)) return FLEXSAE_ERR_UNSUPPORTED;
   if (s->B > ((1LL << 32) - 1) / s->K) return FLEXSAE_ERR_UNSUPPORTED;  // B*K < 2^32
   return FLEXSAE_OK;
 }
@@ -597,7 +598,7 @@ const char *flexsae_status_string(int status) {
     case FLEXSAE_ERR_INVALID_ARGUMENT:
       return "invalid argument (null pointer, non-positive size or unknown dtype)";
     case FLEXSAE_ERR_UNSUPPORTED:
-      return "unsupported size (need F, D, K < 2^31 and B*K < 2^32)";
+      return "unsupported size (need F, K < 2^31, D < 2^29 and B*K < 2^32)";
     case FLEXSAE_ERR_WORKSPACE:
       return "workspace missing, too small or not 256-byte aligned";
     case FLEXSAE_ERR_LAUNCH:

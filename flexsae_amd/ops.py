@@ -92,8 +92,8 @@ def _validate(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, targe
     for name, t in (("indices", indices), ("vals", vals), ("bias", bias), ("target", target)):
         if t.device != dev:
             raise RuntimeError(f"{name} is on {t.device}, weight on {dev}")
-    if B * K >= 2 ** 32 or F >= 2 ** 31 or D >= 2 ** 31:
-        raise ValueError("sizes beyond the kernels' index range: need B*K < 2^32, F < 2^31, D < 2^31")
+    if B * K >= 2 ** 32 or F >= 2 ** 31 or D >= 2 ** 29:
+        raise ValueError("sizes beyond the kernels' index range: need B*K < 2^32, F < 2^31, D < 2^29")
     return B, K, F, D
 
 

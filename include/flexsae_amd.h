@@ -67,7 +67,7 @@ enum {
                                      /* for a unit upstream gradient; multiply dW by grad_out[0]*/
 };
 
-/* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^31; B*K < 2^32. */
+/* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^29; B*K < 2^32. */
 typedef struct {
   int64_t B, K, F, D;
   int32_t weight_dtype, vals_dtype, bias_dtype, target_dtype; /* flexsae_dtype */
