@@ -210,6 +210,15 @@ def main():
     hier_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
     hier_peak = torch.cuda.max_memory_allocated() - base_mem
     Wp.grad = vp.grad = bp.grad = None
+    # the same step with nothing staged between forward and backward (flat memory): forward
+    # kernel + sliced backward
+    stage_budget = flex.ops._hier_stage_bytes
+    flex.set_hier_stage_bytes(0)
+    torch.cuda.reset_peak_memory_stats()
+    flat_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
+    flat_peak = torch.cuda.max_memory_allocated() - base_mem
+    flex.set_hier_stage_bytes(stage_budget)
+    Wp.grad = vp.grad = bp.grad = None
     torch.cuda.reset_peak_memory_stats()
     topk_ms = time_steps(torch, lambda: step(flex.triton_topk_sae_loss), args.steps, args.warmup)
     topk_peak = torch.cuda.max_memory_allocated() - base_mem
@@ -356,6 +365,8 @@ def main():
         "topk": {"ms_per_step": round(topk_ms, 4), "algorithmic_bytes": abytes["topk_step"],
                  "achieved_GBps": round(gbps(abytes["topk_step"], topk_ms), 1)},
         "hier_over_topk_latency": round(hier_ms / topk_ms, 3),
+        "hier_flat_memory_mode": {"ms_per_step": round(flat_ms, 4), "over_topk_latency": round(flat_ms / topk_ms, 3),
+                                  "peak_mem_gib": round(flat_peak / 2 ** 30, 3)},
         "peak_mem_gib": {"hier": round(hier_peak / 2 ** 30, 3), "topk": round(topk_peak / 2 ** 30, 3),
                          "inputs": round(base_mem / 2 ** 30, 3)},
     }
