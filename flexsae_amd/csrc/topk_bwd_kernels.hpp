@@ -5,6 +5,9 @@
 #include "common.hpp"
 #include "segment_kernels.hpp"
 
+#ifndef FLEXSAE_TOPK_ONE_GROUP
+#define FLEXSAE_TOPK_ONE_GROUP 1
+#endif
 #ifndef FLEXSAE_TOPK_NT
 #define FLEXSAE_TOPK_NT true
 #endif
@@ -99,7 +102,10 @@ __device__ __forceinline__ void topk_short_latent(
   const int my_b = static_cast<int>(bv[0]);
   const uint32_t vbits = bv[1];
 
-  raw_vec_t<RT, VEC> buf_a[8], buf_b[8];
+  // two groups of eight rows in flight, or one when a group alone takes 32 registers: the
+  // kernel gains more from another wavefront per SIMD than from the deeper prefetch
+  constexpr bool kTwoGroups = sizeof(raw_vec_t<RT, VEC>) * 8 <= 64 || !FLEXSAE_TOPK_ONE_GROUP;
+  raw_vec_t<RT, VEC> buf_a[8], buf_b[kTwoGroups ? 8 : 1];
   auto issue = [&](raw_vec_t<RT, VEC>(&buf)[8], int j) {
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -108,7 +114,9 @@ __device__ __forceinline__ void topk_short_latent(
     }
   };
   issue(buf_a, 0);
-  if (n > 8) issue(buf_b, 8);
+  if constexpr (kTwoGroups) {
+    if (n > 8) issue(buf_b, 8);
+  }
 
   float w[VEC], acc[VEC];
   unpack_raw<WT, VEC>(wraw, w);
@@ -167,12 +175,19 @@ __device__ __forceinline__ void topk_short_latent(
     const float tot = wave_sum8_transposed(dots);  // lane L: total of slot j + (L & 7)
     if ((lane >> 3) == (j >> 3)) my_dot = tot;
   };
-  for (int j = 0; j < n; j += 16) {
-    consume(buf_a, j);
-    if (j + 16 < n) issue(buf_a, j + 16);
-    if (j + 8 < n) {
-      consume(buf_b, j + 8);
-      if (j + 24 < n) issue(buf_b, j + 24);
+  if constexpr (kTwoGroups) {
+    for (int j = 0; j < n; j += 16) {
+      consume(buf_a, j);
+      if (j + 16 < n) issue(buf_a, j + 16);
+      if (j + 8 < n) {
+        consume(buf_b, j + 8);
+        if (j + 24 < n) issue(buf_b, j + 24);
+      }
+    }
+  } else {
+    for (int j = 0; j < n; j += 8) {
+      consume(buf_a, j);
+      if (j + 8 < n) issue(buf_a, j + 8);
     }
   }
   if (late_scale) {
