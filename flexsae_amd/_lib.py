@@ -66,6 +66,8 @@ SIGNATURES = {
     "flexsae_hier_bwd_atomic": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p]),
     "flexsae_csr_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "flexsae_csr_build": (_int, [_p, _i64, _i64, _i64, _p, _p, _p, _sz, _p, _p]),
+    "flexsae_hier_pair_list_layout": (_int, [_shape_p, ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
+    "flexsae_hier_import_pair_list": (_int, [_shape_p, _p, _p, _p, _sz, _p]),
     "flexsae_topk_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p]),
     "flexsae_topk_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_cast_from_f32": (_int, [_p, _int, _p, _i64, _p]),

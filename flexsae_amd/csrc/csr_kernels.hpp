@@ -210,6 +210,12 @@ __global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__re
   }
 }
 
+__global__ void copy_u32_kernel(uint32_t *__restrict__ dst, const uint32_t *__restrict__ src, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = src[i];
+}
+
 // slot[map[s]] = s: position of every pair in the latent-major list.
 __global__ void csr_inverse_kernel(const uint32_t *__restrict__ map, int64_t n_pairs,
                                    uint32_t *__restrict__ slot) {

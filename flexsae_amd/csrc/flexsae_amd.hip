@@ -732,6 +732,46 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   return launch_status();
 }
 
+int flexsae_hier_pair_list_layout(const flexsae_shape *s, size_t *begin_offset, size_t *map_offset) {
+  const int rc = check_shape(s);
+  if (rc != FLEXSAE_OK) return rc;
+  if (!begin_offset || !map_offset) return FLEXSAE_ERR_INVALID_ARGUMENT;
+  const HierBwdPlan pl = plan_hier_bwd(s);
+  *begin_offset = pl.off_begin;
+  *map_offset = pl.off_map;
+  return FLEXSAE_OK;
+}
+
+int flexsae_hier_import_pair_list(const flexsae_shape *s, const uint32_t *begin, const uint32_t *map,
+                                  void *workspace, size_t workspace_bytes, void *stream) {
+  const int rc = check_shape(s);
+  if (rc != FLEXSAE_OK) return rc;
+  if (!begin || !map) return FLEXSAE_ERR_INVALID_ARGUMENT;
+  if (!aligned(begin, 4) || !aligned(map, 4)) return FLEXSAE_ERR_ALIGNMENT;
+  const HierBwdPlan pl = plan_hier_bwd(s);
+  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, pl.tile))
+    return FLEXSAE_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint8_t *ws = static_cast<uint8_t *>(workspace);
+  uint32_t *ws_begin = reinterpret_cast<uint32_t *>(ws + pl.off_begin);
+  uint32_t *ws_map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
+  const int64_t n_pairs = s->B * s->K;
+  if (ws_begin != begin)
+    hipLaunchKernelGGL(copy_u32_kernel, dim3(grid_for(s->F + 1, 256, 4096)), dim3(256), 0, st, ws_begin, begin,
+                       s->F + 1);
+  if (ws_map != map)
+    hipLaunchKernelGGL(copy_u32_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, ws_map, map, n_pairs);
+  hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, ws_map, n_pairs,
+                     reinterpret_cast<uint32_t *>(ws + pl.off_slot));
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, sc.long_count, static_cast<int64_t>(1), 0u);
+  hipLaunchKernelGGL(seg_find_long_kernel, dim3(grid_for(s->F, 256, 2048)), dim3(256), 0, st, ws_begin, s->F,
+                     sc.long_count, sc.long_list);
+  hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, ws_begin, sc.long_count, sc.long_list,
+                     reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+  return launch_status();
+}
+
 int flexsae_hier_fwd_bwd_supported(const flexsae_shape *s) {
   return check_shape(s) == FLEXSAE_OK && train_supported(s) ? 1 : 0;
 }

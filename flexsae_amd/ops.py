@@ -19,6 +19,7 @@ index checking is switched on.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 from typing import Tuple
@@ -80,7 +81,7 @@ def _validate(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, targe
     if B == 0 or K == 0 or F == 0 or D == 0:
         raise ValueError("empty inputs are not supported (B, K, F, D must all be >= 1)")
     if indices.dtype != torch.int64:
-        raise TypeError(f"indices must be int64, got {indices.dtype}")
+        raise TypeError(f"indices must be int64 (int32 is widened by the public functions), got {indices.dtype}")
     for name, t in (("weight", weight), ("vals", vals), ("bias", bias), ("target", target)):
         if t.dtype not in _DTYPES:
             raise TypeError(f"{name} must be float32, bfloat16 or float16, got {t.dtype}")
@@ -184,6 +185,66 @@ def set_hier_stage_bytes(nbytes: int) -> None:
     _hier_stage_bytes = int(nbytes)
 
 
+# ---- one pair list for both losses ---------------------------------------------------------
+# While a `shared_pair_list()` block is active, the latent-major pair list (begin[F+1], map[B*K])
+# of an `indices` tensor is built by the first backward that needs it and reused by the others.
+_pair_cache = None
+
+
+@contextlib.contextmanager
+def shared_pair_list():
+    """Share the latent-major pair list between losses evaluated on the same ``indices`` tensor.
+
+    Inside the block, the first TopK or hierarchical call that needs the list of an ``indices``
+    tensor builds it; later calls on the same tensor (same storage, unmodified) reuse it instead
+    of rebuilding it, e.g. when a training step evaluates both losses.  Results do not change.
+    The cached lists (and the ``indices`` tensors they belong to) are released when the block ends."""
+    global _pair_cache
+    outer = _pair_cache
+    if outer is None:
+        _pair_cache = {}
+    try:
+        yield
+    finally:
+        _pair_cache = outer
+
+
+def _pair_key(indices: Tensor, F: int):
+    return (indices.data_ptr(), indices._version, tuple(indices.shape), F, indices.device.index)
+
+
+def _pair_lookup(indices: Tensor, F: int):
+    if _pair_cache is None:
+        return None
+    hit = _pair_cache.get(_pair_key(indices, F))
+    return None if hit is None else hit[1:]
+
+
+def _pair_store(indices: Tensor, F: int, begin: Tensor, pair_map: Tensor) -> None:
+    if _pair_cache is not None:
+        # the entry keeps `indices` alive, so its address cannot be handed to another tensor
+        _pair_cache[_pair_key(indices, F)] = (indices, begin, pair_map)
+
+
+def _pair_import(lib, shape, workspace: Tensor, cached) -> None:
+    begin, pair_map = cached
+    rc = lib.flexsae_hier_import_pair_list(ctypes.byref(shape), _ptr(begin), _ptr(pair_map), _ptr(workspace),
+                                           workspace.numel(), _stream())
+    _lib.check(rc, "flexsae_hier_import_pair_list")
+
+
+def _pair_export(lib, shape, workspace: Tensor, indices: Tensor, F: int) -> None:
+    if _pair_cache is None:
+        return
+    ob, om = ctypes.c_size_t(), ctypes.c_size_t()
+    _lib.check(lib.flexsae_hier_pair_list_layout(ctypes.byref(shape), ctypes.byref(ob), ctypes.byref(om)),
+               "flexsae_hier_pair_list_layout")
+    n_pairs = indices.numel()
+    begin = workspace[ob.value: ob.value + (F + 1) * 4].view(torch.int32).clone()
+    pair_map = workspace[om.value: om.value + n_pairs * 4].view(torch.int32).clone()
+    _pair_store(indices, F, begin, pair_map)
+
+
 @torch.library.custom_op("flexsae_amd::hier_bwd", mutates_args=())
 def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
              resid: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
@@ -203,10 +264,17 @@ def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
             ws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
             workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             dW = torch.empty_like(weight)
+            cached = _pair_lookup(indices, F)
+            if cached is not None:
+                _pair_import(lib, shape, workspace, cached)
             rc = lib.flexsae_hier_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(resid),
                                       _ptr(g), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals), _ptr(dbias),
-                                      _ptr(workspace), ws_bytes, 0, _ptr(_flag_for(dev)), _stream())
+                                      _ptr(workspace), ws_bytes,
+                                      _lib.BWD_REUSE_PAIR_LIST if cached is not None else 0,
+                                      _ptr(_flag_for(dev)), _stream())
             _lib.check(rc, "flexsae_hier_bwd")
+            if cached is None:
+                _pair_export(lib, shape, workspace, indices, F)
             return dW, dvals, dbias
         dW_acc = torch.empty((F, D), dtype=torch.float32, device=dev)
         rc = lib.flexsae_hier_bwd_atomic(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals),
@@ -233,13 +301,18 @@ def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
     with torch.cuda.device(dev):
         g = _grad_scalar(grad_out, dev)
         shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
-        begin = torch.empty(F + 1, dtype=torch.int32, device=dev)   # uint32 payload
-        pair_map = torch.empty(B * K, dtype=torch.int32, device=dev)  # uint32 payload
-        ws_bytes = lib.flexsae_csr_workspace_bytes(B, K, F)
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-        rc = lib.flexsae_csr_build(_ptr(indices), B, K, F, _ptr(begin), _ptr(pair_map), _ptr(workspace),
-                                   ws_bytes, _ptr(_flag_for(dev)), _stream())
-        _lib.check(rc, "flexsae_csr_build")
+        cached = _pair_lookup(indices, F)
+        if cached is not None:
+            begin, pair_map = cached
+        else:
+            begin = torch.empty(F + 1, dtype=torch.int32, device=dev)   # uint32 payload
+            pair_map = torch.empty(B * K, dtype=torch.int32, device=dev)  # uint32 payload
+            ws_bytes = lib.flexsae_csr_workspace_bytes(B, K, F)
+            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            rc = lib.flexsae_csr_build(_ptr(indices), B, K, F, _ptr(begin), _ptr(pair_map), _ptr(workspace),
+                                       ws_bytes, _ptr(_flag_for(dev)), _stream())
+            _lib.check(rc, "flexsae_csr_build")
+            _pair_store(indices, F, begin, pair_map)
         dW = torch.empty_like(weight)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
@@ -328,11 +401,16 @@ def hier_train(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
         flag = _flag_for(dev)
+        cached = _pair_lookup(indices, F)
+        if cached is not None:
+            _pair_import(lib, shape, stage, cached)
+        flags = _lib.BWD_SWEEP_ONLY | (_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0)
         rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
                                       _ptr(target), _ptr(loss), None, _DTYPES[weight.dtype], _ptr(dvals),
-                                      _ptr(dbias), _ptr(stage), ws_bytes, _lib.BWD_SWEEP_ONLY, _ptr(flag),
-                                      _stream())
+                                      _ptr(dbias), _ptr(stage), ws_bytes, flags, _ptr(flag), _stream())
         _lib.check(rc, "flexsae_hier_fwd_bwd")
+        if cached is None:
+            _pair_export(lib, shape, stage, indices, F)
         if _check_indices:
             check_index_flag(dev)
     return loss, dvals, dbias, stage
@@ -429,6 +507,8 @@ def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, 
 
     Same name, argument order and meaning as the reference entry point
     (torch-ext/flex_sae/hierarchical_kernels.py:302-309); the kernels underneath are HIP."""
+    if indices.dtype == torch.int32:
+        indices = indices.to(torch.int64)
     needs_grad = torch.is_grad_enabled() and (weight.requires_grad or vals.requires_grad or bias.requires_grad)
     if (needs_grad and _fused_training and weight.dim() == 2 and indices.dim() == 2
             and _train_supported(weight, indices.shape[1]) and _stage_fits(indices, weight)):
@@ -442,4 +522,6 @@ def triton_topk_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, bias: Te
 
     Same name, argument order and meaning as the reference entry point
     (torch-ext/flex_sae/topk_kernels.py:213-223); the kernels underneath are HIP."""
+    if indices.dtype == torch.int32:
+        indices = indices.to(torch.int64)
     return topk_fwd(indices, weight, vals, bias, target)[0]

@@ -197,6 +197,20 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
                       void *stream);
 
 /*
+ * Sharing one pair list between the two losses when both are evaluated on the same `indices`
+ * (the reference rebuilds its map in every embedding_bag_backward call, topk_kernels.py:149-163).
+ * flexsae_hier_pair_list_layout: byte offsets, inside a workspace of flexsae_hier_bwd /
+ *   flexsae_hier_fwd_bwd, of the begin[F+1] and map[B*K] arrays those calls build; after such a
+ *   call, workspace + offset can be handed to flexsae_topk_bwd as they are.
+ * flexsae_hier_import_pair_list: the other direction; copies begin/map (from flexsae_csr_build
+ *   or from another workspace) into `workspace` and derives the rest (slots, hot-latent tables),
+ *   after which flexsae_hier_bwd / flexsae_hier_fwd_bwd can run with FLEXSAE_BWD_REUSE_PAIR_LIST.
+ */
+int flexsae_hier_pair_list_layout(const flexsae_shape *shape, size_t *begin_offset, size_t *map_offset);
+int flexsae_hier_import_pair_list(const flexsae_shape *shape, const uint32_t *begin, const uint32_t *map,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * TopK backward: latent-major segment reduction (no atomics on dW).
  * replaces: aggregate_gradient_for_embedding_kernel and its launch, plus the autograd of
  *           the eager loss tail that produces `gradient` and the bias gradient

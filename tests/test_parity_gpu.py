@@ -463,3 +463,78 @@ def test_opcheck_and_compile(mode):
     assert abs(compiled.item() - 2.0 * eager.item()) <= 1e-6 * abs(eager.item())
     compiled.backward()
     assert W.grad is not None and v.grad is not None and b.grad is not None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("order", ["topk_first", "hier_first"])
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "unfused"])
+def test_shared_pair_list_changes_nothing(order, fused, dtype):
+    """Inside shared_pair_list() the second loss on the same indices reuses the first one's pair
+    list; loss and gradients stay bit-identical to the unshared calls."""
+    args = make_inputs(64, 16, 300, 512, dtype=dtype, seed=77)
+    modes = ["topk", "hier"] if order == "topk_first" else ["hier", "topk"]
+    flex.set_fused_training(fused)
+    try:
+        plain = {m: _run_op(m, args, 0.8) for m in modes}
+        shared = {}
+        idx, W, v, b, t = _to_dev(args)
+        with flex.shared_pair_list():
+            for m in modes:
+                Wm, vm, bm = (x.clone().requires_grad_() for x in (W, v, b))
+                loss = FUSED[m](idx, Wm, vm, bm, t)  # the same indices tensor for both losses
+                loss.backward(torch.tensor(0.8, device=DEV))
+                shared[m] = (loss, Wm.grad, vm.grad, bm.grad)
+            assert len(flex.ops._pair_cache) == 1
+        assert flex.ops._pair_cache is None
+    finally:
+        flex.set_fused_training(True)
+    torch.cuda.synchronize()
+    for m in modes:
+        for a, c in zip(plain[m], shared[m]):
+            assert torch.equal(a, c), m
+
+
+def test_pair_list_import_through_the_c_abi():
+    """flexsae_csr_build -> flexsae_hier_import_pair_list -> flexsae_hier_bwd(REUSE_PAIR_LIST) equals the
+    plain call, and the layout query points at the list a plain call leaves in its workspace."""
+    import ctypes
+    from flexsae_amd import _lib
+    lib = _lib.load()
+    args = _to_dev(make_inputs(40, 24, 90, 640, seed=5))
+    idx, W, v, b, t = args
+    _, _, resid = abi.forward("hier", *args)
+    rc, dW0, dv0, db0 = abi.hier_backward(idx, W, v, resid, 1.25)
+    assert rc == 0
+    sh = abi.shape_of(idx, W, v)
+    rc, begin, mp = abi.csr_build(idx, sh.F)
+    assert rc == 0
+    nbytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), 0)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    assert lib.flexsae_hier_import_pair_list(ctypes.byref(sh), abi.ptr(begin), abi.ptr(mp), abi.ptr(ws), nbytes,
+                                             abi.stream()) == 0
+    dW = torch.full_like(dW0, float("nan"))
+    dv = torch.full_like(dv0, float("nan"))
+    db = torch.full_like(db0, float("nan"))
+    g = torch.tensor([1.25], dtype=torch.float32, device=DEV)
+    rc = lib.flexsae_hier_bwd(ctypes.byref(sh), abi.ptr(idx), abi.ptr(W), abi.ptr(v), abi.ptr(resid), abi.ptr(g),
+                              abi.ptr(dW), abi.DT[torch.float32], abi.ptr(dv), abi.ptr(db), abi.ptr(ws), nbytes,
+                              _lib.BWD_REUSE_PAIR_LIST, None, abi.stream())
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dW, dW0) and torch.equal(dv, dv0) and torch.equal(db, db0)
+    ob, om = ctypes.c_size_t(), ctypes.c_size_t()
+    assert lib.flexsae_hier_pair_list_layout(ctypes.byref(sh), ctypes.byref(ob), ctypes.byref(om)) == 0
+    n_pairs = idx.numel()
+    assert torch.equal(ws[ob.value: ob.value + (sh.F + 1) * 4].view(torch.int32), begin)
+    assert torch.equal(ws[om.value: om.value + n_pairs * 4].view(torch.int32), mp)
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_int32_indices_are_accepted(mode):
+    args = make_inputs(32, 8, 120, 256, seed=12)
+    ref = _run_op(mode, args, 1.0)
+    idx, W, v, b, t = _to_dev(args)
+    W.requires_grad_()
+    loss = FUSED[mode](idx.to(torch.int32), W, v, b, t)
+    loss.backward()
+    assert torch.equal(loss, ref[0]) and torch.equal(W.grad, ref[1])
