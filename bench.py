@@ -39,6 +39,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_k128", choices=sorted(WORKLOADS))
     ap.add_argument("--shape", default="", help="override B,K,F,D of the workload (tuning aid)")
+    ap.add_argument("--no-flat-mode", action="store_true",
+                    help="skip the extra timing of the hierarchical loss in flat-memory mode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU-baseline sample (0 = auto)")
     return ap.parse_args()
@@ -212,12 +214,14 @@ def main():
     Wp.grad = vp.grad = bp.grad = None
     # the same step with nothing staged between forward and backward (flat memory): forward
     # kernel + sliced backward
-    stage_budget = flex.ops._hier_stage_bytes
-    flex.set_hier_stage_bytes(0)
-    torch.cuda.reset_peak_memory_stats()
-    flat_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
-    flat_peak = torch.cuda.max_memory_allocated() - base_mem
-    flex.set_hier_stage_bytes(stage_budget)
+    flat_ms = flat_peak = None
+    if not args.no_flat_mode:
+        stage_budget = flex.ops._hier_stage_bytes
+        flex.set_hier_stage_bytes(0)
+        torch.cuda.reset_peak_memory_stats()
+        flat_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
+        flat_peak = torch.cuda.max_memory_allocated() - base_mem
+        flex.set_hier_stage_bytes(stage_budget)
     Wp.grad = vp.grad = bp.grad = None
     torch.cuda.reset_peak_memory_stats()
     topk_ms = time_steps(torch, lambda: step(flex.triton_topk_sae_loss), args.steps, args.warmup)
@@ -365,8 +369,9 @@ def main():
         "topk": {"ms_per_step": round(topk_ms, 4), "algorithmic_bytes": abytes["topk_step"],
                  "achieved_GBps": round(gbps(abytes["topk_step"], topk_ms), 1)},
         "hier_over_topk_latency": round(hier_ms / topk_ms, 3),
-        "hier_flat_memory_mode": {"ms_per_step": round(flat_ms, 4), "over_topk_latency": round(flat_ms / topk_ms, 3),
-                                  "peak_mem_gib": round(flat_peak / 2 ** 30, 3)},
+        "hier_flat_memory_mode": None if flat_ms is None else {
+            "ms_per_step": round(flat_ms, 4), "over_topk_latency": round(flat_ms / topk_ms, 3),
+            "peak_mem_gib": round(flat_peak / 2 ** 30, 3)},
         "peak_mem_gib": {"hier": round(hier_peak / 2 ** 30, 3), "topk": round(topk_peak / 2 ** 30, 3),
                          "inputs": round(base_mem / 2 ** 30, 3)},
     }
