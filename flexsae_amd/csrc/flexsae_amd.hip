@@ -23,9 +23,6 @@ using namespace flexsae;
 #ifndef FLEXSAE_FWD_U
 #define FLEXSAE_FWD_U 8
 #endif
-#ifndef FLEXSAE_TOPK_U
-#define FLEXSAE_TOPK_U 4
-#endif
 #ifndef FLEXSAE_TOPK_VEC8
 #define FLEXSAE_TOPK_VEC8 1
 #endif
@@ -528,7 +525,7 @@ void launch_topk_slices(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t s
     const int64_t n_short_blocks = ceil_div(s->F, static_cast<int64_t>(kWavesPerBlock));
     const size_t resid_bytes =
         static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * sizeof(typename Traits<RT>::store_t);
-    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, RT, VEC, FLEXSAE_TOPK_U>),
+    hipLaunchKernelGGL((topk_bwd_kernel<WT, GT, RT, VEC>),
                        dim3(kLongBlocks + static_cast<unsigned>(n_short_blocks), static_cast<unsigned>(tps)),
                        dim3(kBlock), 0, st, begin, map, long_count, long_list, chunk_begin,
                        reinterpret_cast<const vec_t<uint32_t, 2> *>(ws + pl.off_slotbv), weight, vals,

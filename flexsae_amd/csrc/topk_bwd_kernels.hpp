@@ -21,7 +21,7 @@ namespace flexsae {
 //                                                      topk_dvals_finalize_kernel adds the tiles up)
 // resid rows (element type RT) are read through the caches: the waves in flight share one
 // B x tile slice of the [B,D] matrix, which has to stay in the 4 MB L2 of every XCD.
-template <typename RT, int VEC, int U>
+template <typename RT, int VEC>
 __device__ __forceinline__ void topk_accumulate_slots(
     const uint32_t *__restrict__ map, const void *__restrict__ vals, int vals_dtype,
     const void *__restrict__ resid, float scale, float *__restrict__ dv_tile, const float (&w)[VEC],
@@ -79,8 +79,8 @@ __device__ __forceinline__ void topk_accumulate_slots(
 
 // One short latent (1 to kSegChunk pairs) for one tile: the pair records of the latent are one
 // contiguous load, the residual rows are gathered through a buffer descriptor (no vector ALU work
-// for addresses) eight at a time with the next eight already requested, and each group of
-// eight shares one transposed wave reduction for the dvals dot products.  Groups are always
+// for addresses) eight at a time (with the next eight already requested when registers allow),
+// and each group of eight shares one transposed wave reduction for the dvals dot products.  Groups are always
 // processed in full: slots past the end re-read the last row (a cache hit) with a val of zero,
 // which keeps the inner code free of branches.  With bf16 weights and a bf16 residual copy the
 // products run on packed pairs (dot2) without unpacking.
@@ -207,7 +207,7 @@ __device__ __forceinline__ void topk_short_latent(
 // B x tile slice of resid (L2-sized); see topk_short_latent.  tile = 64*VEC columns, lane l owning VEC consecutive columns.
 // dW[f, tile] is written exactly once, in the gradient's final dtype; latents without pairs
 // get zeros.
-template <typename WT, typename GT, typename RT, int VEC, int U>
+template <typename WT, typename GT, typename RT, int VEC>
 __global__ __launch_bounds__(256) void topk_bwd_kernel(
     const uint32_t *__restrict__ begin, const uint32_t *__restrict__ map,
     const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(256) void topk_bwd_kernel(
       acc[i] = 0.f;
       if (!active) w[i] = 0.f;
     }
-    topk_accumulate_slots<RT, VEC, U>(map, vals, vals_dtype, resid, scale,
+    topk_accumulate_slots<RT, VEC>(map, vals, vals_dtype, resid, scale,
                                       dv_part + (col0 / (kWave * VEC) + t) * n_pairs, w, c.s0, c.s1, K, D, dsafe,
                                       acc);
     store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
