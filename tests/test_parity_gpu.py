@@ -538,3 +538,22 @@ def test_int32_indices_are_accepted(mode):
     loss = FUSED[mode](idx.to(torch.int32), W, v, b, t)
     loss.backward()
     assert torch.equal(loss, ref[0]) and torch.equal(W.grad, ref[1])
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes(seed):
+    """Seeded random shapes and dtypes, both losses, against the oracle: K below/above the 64-step
+    and 128-step limits of the register-resident paths, D with every vector width, F from a
+    handful of hot latents to mostly unused ones."""
+    rng = np.random.default_rng(1000 + seed)
+    B = int(rng.integers(1, 70))
+    K = int(rng.choice([1, 2, 3, 7, 8, 16, 31, 33, 64, 65, 100, 128, 129, 140]))
+    F = int(rng.choice([1, 2, 5, 40, 300, 2000]))
+    D = int(rng.choice([1, 2, 4, 6, 8, 62, 64, 100, 128, 130, 256, 260, 520, 700]))
+    dtype = [torch.float32, torch.bfloat16, torch.float16][seed % 3]
+    grad_out = float(rng.normal())
+    _announce("random", seed, (B, K, F, D), dtype, grad_out)
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=seed)
+    for mode in ("hier", "topk"):
+        got = _run_op(mode, args, grad_out)
+        _check_against_oracle(mode, args, dtype, grad_out, got, ref_tols=False)
