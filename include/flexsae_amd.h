@@ -106,15 +106,16 @@ int flexsae_topk_fwd(const flexsae_shape *shape, const int64_t *indices, const v
 /*
  * Bytes of workspace flexsae_hier_bwd needs to process `slice_cols` columns of D per pass
  * (rounded up to whole 64*vec-column tiles, capped at D; slice_cols <= 0 asks for the minimum).
- * The workspace holds the latent-major pair list, and per slice column one contribution per
- * (b,k) pair (bf16 for bf16 weights, else fp32): about B*K*slice_cols*sizeof elements.
+ * The workspace holds the latent-major pair list, the per-tile shares of dvals (about
+ * D/128 x B*K fp32), and per slice column one contribution per (b,k) pair (bf16 for bf16 weights,
+ * else fp32): about B*K*slice_cols*sizeof elements.
  */
 size_t flexsae_hier_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slice_cols);
 
 /*
  * HierarchicalTopK backward, two phases per slice of D columns:
  *   sweep   : reverse walk over K per row; stores the per-pair contribution vals_k * S_k of the
- *             slice into the workspace, accumulates dvals and dbias;
+ *             slice into the workspace, and the tile's shares of dvals and dbias;
  *   reduce  : latent-major segment reduction of those contributions (sorted pair list, fp32
  *             accumulation, fixed order) writing dW once in `dW_dtype` -- no atomics on dW, the
  *             result is deterministic, hot latents are split into 64-pair chunks.
@@ -124,8 +125,9 @@ size_t flexsae_hier_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slic
  *           mul_(grad) passes of HierarchicalSAELossFunction.backward and the autograd engine's
  *           cast of the fp32 gradient  (hierarchical_kernels.py:92-187, 230-270, 294-299)
  * in : resid from flexsae_hier_fwd; grad_out device scalar.
- * out: dW[F,D] in dW_dtype (every element written); dvals[B,K] fp32 (zero-filled here unless
- *      FLEXSAE_BWD_OUTPUTS_PREZEROED); dbias[D] fp32 (written, fixed summation order).
+ * out: dW[F,D] in dW_dtype, dvals[B,K] fp32, dbias[D] fp32: every element written once, all
+ *      sums in a fixed order (bit-reproducible); FLEXSAE_BWD_OUTPUTS_PREZEROED is accepted and
+ *      has nothing left to skip.
  */
 int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
                      const void *vals, const float *resid, const float *grad_out, void *dW,
