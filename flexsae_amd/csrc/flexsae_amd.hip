@@ -205,7 +205,7 @@ void zero_f32(float *p, int64_t n, hipStream_t st) {
 }
 
 // Scratch of the pair-list construction, carved out of one workspace:
-// cursor[F] | scan block sums[ceil(F/kScanBlockElems)] | long_count (one aligned slot) |
+// rank[B*K] | scan block sums[ceil(F/kScanBlockElems)] | long_count (one aligned slot) |
 // long_list[B*K/65 + 1]
 struct CsrScratch {
   uint32_t *rank;
