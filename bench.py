@@ -348,7 +348,7 @@ def main():
         "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
                                f"indices {dist}", "B": B, "K": K, "F": F, "D": D,
                    "hier_scratch_mb": scratch >> 20, "fused_training_step": bool(fused),
-                   "hier_stage_mb": int(os.environ.get("FLEXSAE_HIER_STAGE_MB", "4096"))},
+                   "hier_stage_mb": flex.ops.hier_stage_bytes(dev) >> 20},
         "roofline": roofline,
         "step_hbm": {"algorithmic_bytes": abytes["hier_step"],
                      "achieved_GBps": round(gbps(abytes["hier_step"], hier_ms), 1),

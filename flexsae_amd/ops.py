@@ -173,16 +173,31 @@ def set_hier_scratch_bytes(nbytes: int) -> None:
 
 
 # Memory the fused training step may hold between forward and backward: all B*K*D per-pair
-# contributions (2 bytes each for bf16 weights, else 4) plus the pair list.
-_hier_stage_bytes = int(os.environ.get("FLEXSAE_HIER_STAGE_MB", "4096")) << 20
+# contributions (2 bytes each for bf16 weights, else 4) plus the pair list.  Unless set, the
+# budget is one eighth of the device's memory (36 GB on a 288 GB MI355X).
+_hier_stage_bytes = (int(os.environ["FLEXSAE_HIER_STAGE_MB"]) << 20) if "FLEXSAE_HIER_STAGE_MB" in os.environ else None
+_device_stage_default = {}
 
 
-def set_hier_stage_bytes(nbytes: int) -> None:
+def set_hier_stage_bytes(nbytes) -> None:
     """Upper bound (bytes) on what the fused training step keeps alive from forward to backward.
     Calls whose contributions do not fit run the separate forward and sliced backward instead;
-    0 switches the fused step off for every shape."""
+    0 switches the fused step off for every shape (flat memory); None restores the default, one
+    eighth of the device's memory."""
     global _hier_stage_bytes
-    _hier_stage_bytes = int(nbytes)
+    _hier_stage_bytes = None if nbytes is None else int(nbytes)
+
+
+def hier_stage_bytes(device) -> int:
+    """The stage budget in force for tensors on ``device``."""
+    if _hier_stage_bytes is not None:
+        return _hier_stage_bytes
+    index = torch.device(device).index
+    if index is None:
+        index = torch.cuda.current_device()
+    if index not in _device_stage_default:
+        _device_stage_default[index] = torch.cuda.get_device_properties(index).total_memory // 8
+    return _device_stage_default[index]
 
 
 # ---- one pair list for both losses ---------------------------------------------------------
@@ -374,7 +389,7 @@ def _stage_fits(indices: Tensor, weight: Tensor) -> bool:
     B, K = indices.shape
     D = weight.shape[1]
     p_size = 2 if weight.dtype == torch.bfloat16 else 4
-    return B * K * (-(-D // 256) * 256) * p_size <= _hier_stage_bytes
+    return B * K * (-(-D // 256) * 256) * p_size <= hier_stage_bytes(weight.device)
 
 
 def _single_slice_workspace_bytes(lib, shape, D: int) -> int:
