@@ -17,6 +17,14 @@ __global__ void fill_u32_kernel(uint32_t *__restrict__ p, int64_t n, uint32_t va
     p[i] = value;
 }
 
+// Start of a pair-list build: zero the per-latent counters and the long-latent counter.
+__global__ void csr_init_kernel(uint32_t *__restrict__ counts, int64_t n, uint32_t *__restrict__ long_count) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    counts[i] = 0u;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *long_count = 0u;
+}
+
 // counts[f] += 1 for every pair, and rank[p] = the value the counter had before: a position
 // inside the latent's group that is unique but depends on the order the atomics were served in
 // (the groups are sorted afterwards).  Out-of-range indices are flagged and counted as latent 0.

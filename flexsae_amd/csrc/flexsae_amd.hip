@@ -233,10 +233,8 @@ CsrScratch carve_csr_scratch(void *workspace, int64_t F, int64_t n_pairs) {
 void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, uint32_t *begin,
                       uint32_t *map, const CsrScratch &sc, int *status_flag, hipStream_t st) {
   const int64_t n_pairs = B * K;
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(F + 1, 256, 4096)), dim3(256), 0, st, begin,
-                     F + 1, 0u);
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, sc.long_count,
-                     static_cast<int64_t>(1), 0u);
+  hipLaunchKernelGGL(csr_init_kernel, dim3(grid_for(F + 1, 256, 4096)), dim3(256), 0, st, begin, F + 1,
+                     sc.long_count);
   hipLaunchKernelGGL(csr_count_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st,
                      indices, n_pairs, F, begin, sc.rank, status_flag);
   const unsigned scan_blocks = static_cast<unsigned>(ceil_div(F, kScanBlockElems));
@@ -885,8 +883,9 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
   if (static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * 4 > 0xffffffffull) return FLEXSAE_ERR_UNSUPPORTED;
   const TopkBwdPlan pl = plan_topk_bwd(s);
   if (!aligned(begin, 4) || !aligned(map, 4) || !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
-      !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.vec * 4) || !aligned(grad_out, 4) ||
-      !aligned(dW, pl.vec * dtype_size(dW_dtype)) || !aligned(dvals, 16) || !aligned(dbias, 4))
+      !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.resid16 ? 16 : pl.vec * 4) ||
+      !aligned(grad_out, 4) || !aligned(dW, pl.vec * dtype_size(dW_dtype)) || !aligned(dvals, 16) ||
+      !aligned(dbias, 4))
     return FLEXSAE_ERR_ALIGNMENT;
   if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < topk_bwd_bytes(pl, pl.tile))
     return FLEXSAE_ERR_WORKSPACE;
@@ -906,16 +905,15 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
                      reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
   const float coef =
       static_cast<float>(2.0 / (static_cast<double>(s->B) * static_cast<double>(s->D)));
-  hipLaunchKernelGGL(topk_slot_records_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map, vals,
-                     s->vals_dtype, s->B * s->K, static_cast<int>(s->K),
-                     reinterpret_cast<vec_t<uint32_t, 2> *>(ws + pl.off_slotbv));
-  const void *gather_src = resid;
-  if (pl.resid16) {
-    void *r16 = ws + pl.off_resid16;
-    const int64_t n = s->B * s->D;
-    hipLaunchKernelGGL(cast_from_f32_kernel<bf16_t>, dim3(grid_for(ceil_div(n, 4), 256, 1 << 16)), dim3(256), 0,
-                       st, r16, resid, n);
-    gather_src = r16;
+  // per-pair records and, for bf16 weights, the bf16 copy of the residual: one launch
+  const void *gather_src = pl.resid16 ? static_cast<const void *>(ws + pl.off_resid16) : resid;
+  {
+    const int64_t n_resid = pl.resid16 ? s->B * s->D : 0;
+    const int64_t work = s->B * s->K > ceil_div(n_resid, 4) ? s->B * s->K : ceil_div(n_resid, 4);
+    hipLaunchKernelGGL(topk_prepare_kernel, dim3(grid_for(work, 256, 1 << 16)), dim3(256), 0, st, map, vals,
+                       s->vals_dtype, s->B * s->K, static_cast<int>(s->K),
+                       reinterpret_cast<vec_t<uint32_t, 2> *>(ws + pl.off_slotbv), resid, n_resid,
+                       pl.resid16 ? static_cast<void *>(ws + pl.off_resid16) : nullptr);
   }
   if (pl.vec == 8) {
     launch_topk_slices_g<bf16_t, bf16_t, 8>(s, pl, slice_w, begin, map, weight, vals, gather_src, grad_out, coef,

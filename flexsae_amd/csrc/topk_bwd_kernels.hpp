@@ -282,18 +282,32 @@ __global__ void topk_dvals_finalize_kernel(const uint32_t *__restrict__ map,
   }
 }
 
-// slot_bv[s] = (batch row, val as fp32 bits) of the pair in slot s of the latent-major list: what
-// the pipelined backward reads per pair, contiguous per latent instead of scattered over vals.
-__global__ void topk_slot_records_kernel(const uint32_t *__restrict__ map, const void *__restrict__ vals,
-                                         int vals_dtype, int64_t n_pairs, int K,
-                                         vec_t<uint32_t, 2> *__restrict__ slot_bv) {
+// Preparation of a TopK backward, one launch:
+//   slot_bv[s] = (batch row, val as fp32 bits) of the pair in slot s of the latent-major list: what
+//     the backward reads per pair, contiguous per latent instead of scattered over vals;
+//   resid16[i] = bf16(resid[i]) for i < n_resid (n_resid = 0: no copy wanted).
+__global__ void topk_prepare_kernel(const uint32_t *__restrict__ map, const void *__restrict__ vals,
+                                    int vals_dtype, int64_t n_pairs, int K,
+                                    vec_t<uint32_t, 2> *__restrict__ slot_bv, const float *__restrict__ resid,
+                                    int64_t n_resid, void *__restrict__ resid16) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t s = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; s < n_pairs; s += stride) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  for (int64_t s = tid; s < n_pairs; s += stride) {
     const uint32_t p = map[s];
     vec_t<uint32_t, 2> r;
     r[0] = p / static_cast<uint32_t>(K);
     r[1] = __float_as_uint(load_scalar(vals, vals_dtype, p));
     slot_bv[s] = r;
+  }
+  const int64_t n4 = n_resid >> 2;
+  for (int64_t i = tid; i < n4; i += stride) {
+    float x[4];
+    load_vec<float, 4>(resid, i * 4, x);
+    store_vec<bf16_t, 4>(resid16, i * 4, x);
+  }
+  for (int64_t i = (n4 << 2) + tid; i < n_resid; i += stride) {
+    float x[1] = {resid[i]};
+    store_vec<bf16_t, 1>(resid16, i, x);
   }
 }
 
