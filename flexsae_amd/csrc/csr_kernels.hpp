@@ -194,12 +194,14 @@ __device__ __forceinline__ void block_bitonic_sort(Ptr a, uint32_t n) {
 }
 
 // Long groups (more than 64 pairs): one block per group, striding over the list.  Groups of up
-// to kSortLdsElems pairs are sorted in LDS, longer ones in place in global memory.
+// to kSortLdsElems pairs are sorted in LDS, longer ones in place in global memory.  With `slot`
+// given, the positions of the group's pairs are written there as well.
 constexpr uint32_t kSortLdsElems = 8192;
 __global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
                                                             uint32_t *__restrict__ map,
                                                             const uint32_t *__restrict__ long_count,
-                                                            const uint32_t *__restrict__ long_list) {
+                                                            const uint32_t *__restrict__ long_list,
+                                                            uint32_t *__restrict__ slot) {
   __shared__ uint32_t buf[kSortLdsElems];
   const uint32_t n_long = *long_count;
   for (uint32_t w = blockIdx.x; w < n_long; w += gridDim.x) {
@@ -210,10 +212,207 @@ __global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__re
       for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) buf[i] = a[i];
       __syncthreads();
       block_bitonic_sort(buf, n);
-      for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) a[i] = buf[i];
+      for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+        a[i] = buf[i];
+        if (slot) slot[buf[i]] = begin[f] + i;
+      }
       __syncthreads();
     } else {
-      block_bitonic_sort(a, n);
+      block_bitonic_sort(a, n);  // ends with a barrier
+      if (slot)
+        for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) slot[a[i]] = begin[f] + i;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Bucketed construction (the default): the latents are cut into buckets of 2^shift consecutive
+// ids, sized so that a bucket holds a few thousand pairs.  csr_bucket_count_kernel counts, for
+// every chunk of consecutive pairs, how many fall into each bucket (LDS atomics only); an
+// exclusive scan of that table (bucket-major) gives every (bucket, chunk) its place;
+// csr_bucket_scatter_kernel moves (latent within bucket, pair id) there; csr_bucket_sort_kernel
+// then finishes one bucket per block inside the LDS: per-latent counts -> begin[], placement,
+// and a rank sort of every group, so that map[] comes out ascending inside each latent and
+// slot[] (its inverse) is written on the way.  No atomics reach memory except one per latent
+// with more than 64 pairs (appended to long_list; csr_sort_long_kernel sorts those groups).
+// ---------------------------------------------------------------------------------
+constexpr int kBucketThreads = 256;
+constexpr int kBucketMaxBuckets = 8192;  // LDS counters of the count / scatter kernels
+constexpr int kSortThreads = 512;
+constexpr int kSortMaxLatents = 4096;    // latents per bucket (2^shift) at most
+constexpr int kSortCap = 8192;           // pairs of a bucket that are sorted inside the LDS
+
+__global__ __launch_bounds__(kBucketThreads) void csr_bucket_count_kernel(
+    const int64_t *__restrict__ indices, int64_t n_pairs, int64_t F, int shift, uint32_t n_buckets,
+    int64_t chunk, uint32_t n_chunks, uint32_t *__restrict__ table, uint32_t *__restrict__ long_count,
+    int *status_flag) {
+  __shared__ uint32_t hist[kBucketMaxBuckets];
+  for (uint32_t q = threadIdx.x; q < n_buckets; q += kBucketThreads) hist[q] = 0u;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *long_count = 0u;
+  __syncthreads();
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * chunk;
+  const int64_t p1 = (p0 + chunk) < n_pairs ? (p0 + chunk) : n_pairs;
+  for (int64_t p = p0 + threadIdx.x; p < p1; p += kBucketThreads) {
+    int64_t f = indices[p];
+    if (static_cast<uint64_t>(f) >= static_cast<uint64_t>(F)) {
+      if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
+      f = 0;
+    }
+    atomicAdd(&hist[f >> shift], 1u);
+  }
+  __syncthreads();
+  for (uint32_t q = threadIdx.x; q < n_buckets; q += kBucketThreads)
+    table[static_cast<size_t>(q) * n_chunks + blockIdx.x] = hist[q];
+}
+
+// tmp[place] = (latent within its bucket) << 32 | pair id; inside one (bucket, chunk) cell the
+// order is that of the LDS atomics, which the sort kernel removes.
+__global__ __launch_bounds__(kBucketThreads) void csr_bucket_scatter_kernel(
+    const int64_t *__restrict__ indices, int64_t n_pairs, int64_t F, int shift, uint32_t n_buckets,
+    int64_t chunk, uint32_t n_chunks, const uint32_t *__restrict__ table, uint64_t *__restrict__ tmp) {
+  __shared__ uint32_t cursor[kBucketMaxBuckets];
+  for (uint32_t q = threadIdx.x; q < n_buckets; q += kBucketThreads)
+    cursor[q] = table[static_cast<size_t>(q) * n_chunks + blockIdx.x];
+  __syncthreads();
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * chunk;
+  const int64_t p1 = (p0 + chunk) < n_pairs ? (p0 + chunk) : n_pairs;
+  const int64_t mask = (static_cast<int64_t>(1) << shift) - 1;
+  for (int64_t p = p0 + threadIdx.x; p < p1; p += kBucketThreads) {
+    int64_t f = indices[p];
+    if (static_cast<uint64_t>(f) >= static_cast<uint64_t>(F)) f = 0;
+    const uint32_t place = atomicAdd(&cursor[f >> shift], 1u);
+    tmp[place] = (static_cast<uint64_t>(f & mask) << 32) | static_cast<uint64_t>(static_cast<uint32_t>(p));
+  }
+}
+
+// Exclusive scan of a[0..n) in LDS by a whole block of kSortThreads threads (n <= 8 per thread);
+// every thread owns 8 consecutive entries.  Ends with a barrier.
+__device__ __forceinline__ void block_exclusive_scan_lds(uint32_t *a, uint32_t n, uint32_t *wave_tot) {
+  constexpr int PER = kSortMaxLatents / kSortThreads;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid >> 6;
+  uint32_t x[PER];
+  uint32_t tsum = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const uint32_t k = static_cast<uint32_t>(tid) * PER + i;
+    x[i] = (k < n) ? a[k] : 0u;
+    tsum += x[i];
+  }
+  uint32_t inc = tsum;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const uint32_t y = __shfl_up(inc, off, kWave);
+    if (lane >= off) inc += y;
+  }
+  if (lane == kWave - 1) wave_tot[wv] = inc;
+  __syncthreads();
+  uint32_t run = inc - tsum;
+  for (int w = 0; w < wv; ++w) run += wave_tot[w];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const uint32_t k = static_cast<uint32_t>(tid) * PER + i;
+    if (k < n) a[k] = run;
+    run += x[i];
+  }
+  __syncthreads();
+}
+
+// One block per bucket.  `map` and `slot` are written here and, in the large-bucket path, map
+// is read back by other wavefronts of the same block after a barrier.  cnt[] holds, in turn, the
+// per-latent counts, the first position of every latent (after the scan) and the end of every
+// latent's group (after the placement, whose atomics advance it).
+__global__ __launch_bounds__(kSortThreads) void csr_bucket_sort_kernel(
+    const uint64_t *__restrict__ tmp, const uint32_t *__restrict__ table, uint32_t n_chunks, int shift,
+    int64_t F, uint32_t *begin, uint32_t *map, uint32_t *slot, uint32_t *long_count, uint32_t *long_list) {
+  __shared__ uint32_t cnt[kSortMaxLatents + 1];
+  __shared__ uint32_t ids[kSortCap];  // pair ids grouped by latent
+  __shared__ uint32_t wave_tot[kSortThreads / kWave];
+  __shared__ uint32_t any_long;
+  const int tid = threadIdx.x;
+  const uint32_t q = blockIdx.x;
+  const uint32_t lpb = 1u << shift;
+  const int64_t f0 = static_cast<int64_t>(q) << shift;
+  const uint32_t nlat = (F - f0) < static_cast<int64_t>(lpb) ? static_cast<uint32_t>(F - f0) : lpb;
+  const uint32_t base = table[static_cast<size_t>(q) * n_chunks];
+  const uint32_t end = table[static_cast<size_t>(q + 1) * n_chunks];  // the scan's total after the last bucket
+  const uint32_t n = end - base;
+  const bool in_lds = n <= static_cast<uint32_t>(kSortCap);
+  for (uint32_t k = tid; k <= lpb; k += kSortThreads) cnt[k] = 0u;
+  if (tid == 0) any_long = 0u;
+  __syncthreads();
+  for (uint64_t i = tid; i < n; i += kSortThreads) atomicAdd(&cnt[static_cast<uint32_t>(tmp[base + i] >> 32)], 1u);
+  __syncthreads();
+  block_exclusive_scan_lds(cnt, lpb, wave_tot);
+  if (tid == 0) cnt[lpb] = n;
+  __syncthreads();
+  for (uint32_t k = tid; k < nlat; k += kSortThreads) {
+    begin[f0 + k] = base + cnt[k];
+    if (cnt[k + 1] - cnt[k] > static_cast<uint32_t>(kWave)) {
+      long_list[atomicAdd(long_count, 1u)] = static_cast<uint32_t>(f0 + k);
+      any_long = 1u;
+    }
+  }
+  if (q == gridDim.x - 1 && tid == 0) begin[F] = end;
+  __syncthreads();
+  // placement: inside a group the order is that of the atomics
+  for (uint64_t i = tid; i < n; i += kSortThreads) {
+    const uint64_t kv = tmp[base + i];
+    const uint32_t place = atomicAdd(&cnt[static_cast<uint32_t>(kv >> 32)], 1u);
+    if (in_lds)
+      ids[place] = static_cast<uint32_t>(kv);
+    else
+      map[base + place] = static_cast<uint32_t>(kv);
+  }
+  __syncthreads();  // also makes the block's own writes to map visible to all its wavefronts
+  // from here: the group of latent k is [k ? cnt[k-1] : 0, cnt[k])
+
+  if (in_lds) {
+    // every pair finds its rank inside its group by counting the smaller ids
+    for (uint64_t i = tid; i < n; i += kSortThreads) {
+      const uint64_t kv = tmp[base + i];
+      const uint32_t key = static_cast<uint32_t>(kv >> 32), id = static_cast<uint32_t>(kv);
+      const uint32_t s0 = key ? cnt[key - 1] : 0u, len = cnt[key] - s0;
+      if (len > static_cast<uint32_t>(kWave)) continue;
+      uint32_t rank = 0;
+      for (uint32_t j = 0; j < len; ++j) rank += (ids[s0 + j] < id) ? 1u : 0u;
+      map[base + s0 + rank] = id;
+      if (slot) slot[id] = base + s0 + rank;
+    }
+    if (any_long) {
+      // groups of more than 64 pairs go out as they are: csr_sort_long_kernel orders them and
+      // writes their slots.  The latent of position j is found by bisection over the group ends.
+      for (uint32_t j = tid; j < n; j += kSortThreads) {  // n <= kSortCap here
+        uint32_t lo = 0, hi = lpb - 1;  // smallest k with cnt[k] > j
+        while (lo < hi) {
+          const uint32_t mid = (lo + hi) >> 1;
+          if (cnt[mid] > j)
+            hi = mid;
+          else
+            lo = mid + 1;
+        }
+        const uint32_t s0 = lo ? cnt[lo - 1] : 0u;
+        if (cnt[lo] - s0 > static_cast<uint32_t>(kWave)) map[base + j] = ids[j];
+      }
+    }
+    return;
+  }
+
+  // A bucket too large for the LDS (hot latents): the groups were placed in map; one wavefront
+  // per latent rank-sorts its group there.
+  const int lane = tid & (kWave - 1);
+  for (uint32_t k = tid >> 6; k < nlat; k += kSortThreads / kWave) {
+    const uint32_t s0 = k ? cnt[k - 1] : 0u, len = cnt[k] - s0;
+    if (len == 0 || len > static_cast<uint32_t>(kWave)) continue;
+    const bool have = static_cast<uint32_t>(lane) < len;
+    const uint32_t x = have ? map[base + s0 + lane] : 0xffffffffu;
+    uint32_t rank = 0;
+    for (uint32_t j = 0; j < len; ++j) {
+      const uint32_t y = static_cast<uint32_t>(bcast_i32(static_cast<int>(x), static_cast<int>(j)));
+      rank += (y < x) ? 1u : 0u;
+    }
+    if (have) {
+      map[base + s0 + rank] = x;  // every lane read its element before any lane writes
+      if (slot) slot[x] = base + s0 + rank;
     }
   }
 }

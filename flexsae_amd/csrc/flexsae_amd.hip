@@ -204,35 +204,112 @@ void zero_f32(float *p, int64_t n, hipStream_t st) {
                      p, n);
 }
 
+// How a pair list is built for a given problem size.  The bucketed construction serves every
+// size whose bucket count fits the LDS counters of its kernels; beyond that (more than
+// kBucketMaxBuckets * kSortMaxLatents latents) the list is built with one memory atomic per pair.
+struct CsrPlan {
+  bool bucketed;
+  int shift;           // a bucket is 2^shift consecutive latents
+  uint32_t n_buckets;
+  int64_t chunk;       // consecutive pairs counted by one block
+  uint32_t n_chunks;
+  size_t table_len;    // n_buckets * n_chunks (+1 entry for the total)
+};
+
+CsrPlan plan_csr(int64_t n_pairs, int64_t F) {
+  CsrPlan p;
+  // latents per bucket: about 2048 pairs per bucket on average, a power of two
+  int shift = 0;
+  while (shift < 12 && (static_cast<int64_t>(2) << shift) * n_pairs <= 2048 * F) ++shift;
+  static_assert((1 << 12) == kSortMaxLatents, "shift limit follows the LDS counters of the sort kernel");
+  while (shift < 12 && ceil_div(F, static_cast<int64_t>(1) << shift) > kBucketMaxBuckets) ++shift;
+  p.shift = shift;
+  const int64_t n_buckets = ceil_div(F, static_cast<int64_t>(1) << shift);
+  p.bucketed = n_buckets <= kBucketMaxBuckets;
+  p.n_buckets = static_cast<uint32_t>(p.bucketed ? n_buckets : 0);
+  p.chunk = 2048;
+  while (p.bucketed && ceil_div(n_pairs, p.chunk) * n_buckets > (static_cast<int64_t>(1) << 22)) p.chunk *= 2;
+  p.n_chunks = static_cast<uint32_t>(ceil_div(n_pairs, p.chunk));
+  p.table_len = p.bucketed ? static_cast<size_t>(n_buckets) * p.n_chunks : 0;
+  return p;
+}
+
 // Scratch of the pair-list construction, carved out of one workspace:
-// rank[B*K] | scan block sums[ceil(F/kScanBlockElems)] | long_count (one aligned slot) |
-// long_list[B*K/65 + 1]
+//   bucketed: tmp[B*K] u64 | table[table_len + 1] | scan block sums | long_count (one aligned
+//             slot) | long_list[B*K/65 + 1]
+//   atomic:   rank[B*K] u32 | scan block sums[ceil(F/kScanBlockElems)] | long_count | long_list
 struct CsrScratch {
+  CsrPlan plan;
+  uint64_t *tmp;
+  uint32_t *table;
   uint32_t *rank;
   uint32_t *block_sums;
   uint32_t *long_count;
   uint32_t *long_list;
 };
 
-size_t csr_scan_sums_bytes(int64_t F) {
-  return round_up(static_cast<size_t>(ceil_div(F, kScanBlockElems)) * 4, kAlign);
+size_t csr_scan_sums_bytes(int64_t n) {
+  return round_up(static_cast<size_t>(ceil_div(n, kScanBlockElems)) * 4, kAlign);
+}
+
+size_t csr_scratch_bytes(int64_t n_pairs, int64_t F, CsrScratch *sc, uint8_t *ws) {
+  const CsrPlan pl = plan_csr(n_pairs, F);
+  size_t off = 0;
+  if (sc) {
+    sc->plan = pl;
+    sc->tmp = nullptr;
+    sc->table = nullptr;
+    sc->rank = nullptr;
+  }
+  if (pl.bucketed) {
+    if (sc) sc->tmp = reinterpret_cast<uint64_t *>(ws + off);
+    off += round_up(static_cast<size_t>(n_pairs) * 8, kAlign);
+    if (sc) sc->table = reinterpret_cast<uint32_t *>(ws + off);
+    off += round_up((pl.table_len + 1) * 4, kAlign);
+    if (sc) sc->block_sums = reinterpret_cast<uint32_t *>(ws + off);
+    off += csr_scan_sums_bytes(static_cast<int64_t>(pl.table_len));
+  } else {
+    if (sc) sc->rank = reinterpret_cast<uint32_t *>(ws + off);
+    off += round_up(static_cast<size_t>(n_pairs) * 4, kAlign);
+    if (sc) sc->block_sums = reinterpret_cast<uint32_t *>(ws + off);
+    off += csr_scan_sums_bytes(F);
+  }
+  if (sc) sc->long_count = reinterpret_cast<uint32_t *>(ws + off);
+  off += kAlign;
+  if (sc) sc->long_list = reinterpret_cast<uint32_t *>(ws + off);
+  off += round_up((static_cast<size_t>(n_pairs) / 65 + 1) * 4, kAlign);
+  return off;
 }
 
 CsrScratch carve_csr_scratch(void *workspace, int64_t F, int64_t n_pairs) {
-  uint8_t *ws = static_cast<uint8_t *>(workspace);
   CsrScratch sc;
-  sc.rank = reinterpret_cast<uint32_t *>(ws);
-  ws += round_up(static_cast<size_t>(n_pairs) * 4, kAlign);
-  sc.block_sums = reinterpret_cast<uint32_t *>(ws);
-  ws += csr_scan_sums_bytes(F);
-  sc.long_count = reinterpret_cast<uint32_t *>(ws);
-  sc.long_list = reinterpret_cast<uint32_t *>(ws + kAlign);
+  csr_scratch_bytes(n_pairs, F, &sc, static_cast<uint8_t *>(workspace));
   return sc;
 }
 
+// begin[F+1], map[B*K] and, when `slot` is given, its inverse slot[B*K]; leaves the list of
+// latents with more than 64 pairs in sc.long_list / sc.long_count.
 void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, uint32_t *begin,
-                      uint32_t *map, const CsrScratch &sc, int *status_flag, hipStream_t st) {
+                      uint32_t *map, uint32_t *slot, const CsrScratch &sc, int *status_flag, hipStream_t st) {
   const int64_t n_pairs = B * K;
+  const CsrPlan &pl = sc.plan;
+  if (pl.bucketed) {
+    hipLaunchKernelGGL(csr_bucket_count_kernel, dim3(pl.n_chunks), dim3(kBucketThreads), 0, st, indices, n_pairs,
+                       F, pl.shift, pl.n_buckets, pl.chunk, pl.n_chunks, sc.table, sc.long_count, status_flag);
+    const int64_t len = static_cast<int64_t>(pl.table_len);
+    const unsigned scan_blocks = static_cast<unsigned>(ceil_div(len, kScanBlockElems));
+    hipLaunchKernelGGL(csr_scan_sums_kernel, dim3(scan_blocks), dim3(kScanThreads), 0, st, sc.table, len,
+                       sc.block_sums);
+    hipLaunchKernelGGL(csr_scan_apply_kernel, dim3(scan_blocks), dim3(kScanThreads), 0, st, sc.table, len,
+                       sc.block_sums);
+    hipLaunchKernelGGL(csr_bucket_scatter_kernel, dim3(pl.n_chunks), dim3(kBucketThreads), 0, st, indices,
+                       n_pairs, F, pl.shift, pl.n_buckets, pl.chunk, pl.n_chunks, sc.table, sc.tmp);
+    hipLaunchKernelGGL(csr_bucket_sort_kernel, dim3(pl.n_buckets), dim3(kSortThreads), 0, st, sc.tmp, sc.table,
+                       pl.n_chunks, pl.shift, F, begin, map, slot, sc.long_count, sc.long_list);
+    hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(256), 0, st, begin, map, sc.long_count,
+                       sc.long_list, slot);
+    return;
+  }
   hipLaunchKernelGGL(csr_init_kernel, dim3(grid_for(F + 1, 256, 4096)), dim3(256), 0, st, begin, F + 1,
                      sc.long_count);
   hipLaunchKernelGGL(csr_count_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st,
@@ -248,7 +325,10 @@ void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
                      dim3(static_cast<unsigned>(ceil_div(F, kWavesPerBlock))), dim3(kBlock), 0, st,
                      begin, map, F, sc.long_count, sc.long_list);
   hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(256), 0, st, begin, map, sc.long_count,
-                     sc.long_list);
+                     sc.long_list, static_cast<uint32_t *>(nullptr));
+  if (slot)
+    hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, map, n_pairs,
+                       slot);
 }
 
 // ---- two-phase hierarchical backward: workspace plan -----------------------------------
@@ -706,9 +786,8 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
-    csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
-    hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
-                       s->B * s->K, reinterpret_cast<uint32_t *>(ws + pl.off_slot));
+    csr_build_launch(indices, s->B, s->K, s->F, begin, map, reinterpret_cast<uint32_t *>(ws + pl.off_slot), sc,
+                     status_flag, st);
     hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
                        sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
   }
@@ -801,9 +880,8 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   uint32_t *map = reinterpret_cast<uint32_t *>(ws + pl.off_map);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
-    csr_build_launch(indices, s->B, s->K, s->F, begin, map, sc, status_flag, st);
-    hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, map,
-                       s->B * s->K, reinterpret_cast<uint32_t *>(ws + pl.off_slot));
+    csr_build_launch(indices, s->B, s->K, s->F, begin, map, reinterpret_cast<uint32_t *>(ws + pl.off_slot), sc,
+                     status_flag, st);
     hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
                        sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
   }
@@ -843,9 +921,8 @@ int flexsae_scale(void *dst, const void *src, int dtype, int64_t n, const float 
 
 size_t flexsae_csr_workspace_bytes(int64_t B, int64_t K, int64_t F) {
   if (B <= 0 || K <= 0 || F <= 0) return 0;
-  // rank[B*K] | scan block sums | long_count (padded) | long_list[B*K/65 + 1]
-  return round_up(static_cast<size_t>(B) * static_cast<size_t>(K) * 4, kAlign) + csr_scan_sums_bytes(F) + kAlign +
-         round_up((static_cast<size_t>(B) * static_cast<size_t>(K) / 65 + 1) * 4, kAlign);
+  if (B > ((1LL << 32) - 1) / K) return 0;
+  return csr_scratch_bytes(B * K, F, nullptr, nullptr);
 }
 
 int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, uint32_t *begin,
@@ -858,7 +935,7 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
       !aligned(workspace, kAlign))
     return FLEXSAE_ERR_WORKSPACE;
   const CsrScratch sc = carve_csr_scratch(workspace, F, B * K);
-  csr_build_launch(indices, B, K, F, begin, map, sc, status_flag, static_cast<hipStream_t>(stream));
+  csr_build_launch(indices, B, K, F, begin, map, nullptr, sc, status_flag, static_cast<hipStream_t>(stream));
   return launch_status();
 }
 

@@ -190,7 +190,8 @@ size_t flexsae_csr_workspace_bytes(int64_t B, int64_t K, int64_t F);
  * Latent-major pair list for the TopK backward: begin[F+1] (exclusive prefix of
  * the per-latent pair counts, begin[F] = B*K) and map[B*K] holding pair ids
  * p = b*K + t grouped by latent, ascending inside a group (a stable counting
- * sort, so the result is deterministic).
+ * sort, so the result is deterministic).  Built as a bucketed counting sort whose atomics stay
+ * in the LDS; with more than 8192*4096 latents, with one memory atomic per pair.
  * replaces: count_per_embedding_kernel, count.cumsum(0), map_embeddings_and_outputs_kernel
  *           (topk_kernels.py:71-94, 149-163; there the order inside a group is racy)
  */

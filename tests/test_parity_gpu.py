@@ -206,12 +206,20 @@ def test_gather_addressing_is_exact(mode, dtype):
 
 
 @pytest.mark.parametrize("shape", [(4, 8, 16), (37, 16, 5), (64, 32, 4096), (192, 256, 512), (300, 70, 3),
-                                   (128, 64, 100000), (2048, 33, 1)])
+                                   (128, 64, 100000), (2048, 33, 1), (4096, 128, 65536), (1000, 100, 700),
+                                   (64, 16, (1 << 25)), (64, 16, (1 << 25) + 7), (3000, 40, 9000, "skew")])
 def test_pair_list_bit_exact(shape):
-    """begin/map equal the stable counting sort (oracle = numpy argsort(kind='stable'))."""
-    B, K, F = shape
+    """begin/map equal the stable counting sort (oracle = numpy argsort(kind='stable')).  The shapes cover
+    one bucket and many, buckets sorted in the LDS and buckets too large for it, latents with more than 64
+    pairs, the largest bucket count, and (F above 2^25) the construction with memory atomics."""
+    B, K, F = shape[:3]
     _announce("csr", shape)
-    idx = torch.randint(0, F, (B, K), generator=torch.Generator().manual_seed(B + K + F))
+    g = torch.Generator().manual_seed(B + K + F)
+    if len(shape) > 3:  # a few hot latents next to a long uniform tail
+        hot = torch.randint(0, 12, (B, K), generator=g) * 613 % F
+        idx = torch.where(torch.rand(B, K, generator=g) < 0.4, hot, torch.randint(0, F, (B, K), generator=g))
+    else:
+        idx = torch.randint(0, F, (B, K), generator=g)
     rbegin, rmap = oracle.csr(idx, F)
     for _ in range(2):  # twice: the result may not depend on how the atomics were served
         rc, begin, mp = abi.csr_build(idx.to(DEV), F)
