@@ -18,7 +18,7 @@ using namespace flexsae;
 #define FLEXSAE_SWEEP_U 16
 #endif
 #ifndef FLEXSAE_REDUCE_U
-#define FLEXSAE_REDUCE_U 8
+#define FLEXSAE_REDUCE_U 4
 #endif
 #ifndef FLEXSAE_FWD_U
 #define FLEXSAE_FWD_U 8
@@ -476,7 +476,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                          s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F,
                          D);
     if (!do_reduce) continue;
-    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(s->F, kWavesPerBlock));
+    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(s->F * tps, kWavesPerBlock));
     hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock),
                        0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, s->F,
                        kLongBlocks, tps, static_cast<int>(col0), sw, D);

@@ -16,23 +16,24 @@ namespace flexsae {
 constexpr int kSegChunk = 64;  // rows per chunk; groups longer than this count as "long"
 
 // acc += sum of rows [r0, r0+n) of X (row stride `ld` elements) over the lane's VEC columns at pc.
-// Rows are fetched U at a time; a group that reaches past the end re-reads the last row (a cache
-// hit) instead of falling back to one load at a time, so short groups keep all loads in flight.
+// Rows are fetched up to U at a time; n is uniform over the wavefront, so the tests around the
+// loads are scalar branches and a short group issues exactly its own loads, all in flight at once.
 template <typename PT, int VEC, int U, bool NT = false>
 __device__ __forceinline__ void accumulate_rows(const void *__restrict__ X, int64_t r0, int n,
                                                 int64_t ld, int pc, float (&acc)[VEC]) {
   for (int j = 0; j < n; j += U) {
-    float x[U][VEC];
+    raw_vec_t<PT, VEC> raw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int jj = (j + u) < n ? (j + u) : (n - 1);
-      unpack_raw<PT, VEC>(load_raw<PT, VEC, NT>(X, (r0 + jj) * ld + pc), x[u]);
+      if (j + u < n) raw[u] = load_raw<PT, VEC, NT>(X, (r0 + j + u) * ld + pc);  // uniform
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (j + u < n) {  // uniform
+        float x[VEC];
+        unpack_raw<PT, VEC>(raw[u], x);
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) acc[i] += x[u][i];
+        for (int i = 0; i < VEC; ++i) acc[i] += x[i];
       }
     }
   }
@@ -68,8 +69,8 @@ __device__ __forceinline__ LongChunk seg_decode_chunk(const uint32_t *__restrict
 // whose length is only known on the device.  seg_reduce_long_finalize_kernel (next launch)
 // combines the partials in chunk order.  These blocks come first so that hot latents start
 // at once and overlap with the bulk of the work.
-// Remaining blocks: one wavefront per latent walks the tiles of the slice (64*VEC columns
-// each); latents without rows get zeros; latents with more than kSegChunk rows are skipped.
+// Remaining blocks: one wavefront per (latent, tile of 64*VEC columns of the slice); latents
+// without rows get zeros; latents with more than kSegChunk rows are skipped.
 template <typename PT, typename GT, int VEC, int U>
 __global__ __launch_bounds__(256) void seg_reduce_kernel(
     const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
@@ -79,25 +80,26 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
     int slice_w, int D) {
   const int lane = lane_id();
   if (blockIdx.x >= n_long_blocks) {
-    const int64_t f = static_cast<int64_t>(blockIdx.x - n_long_blocks) * (blockDim.x >> 6) + wave_in_block();
+    // one wavefront per (latent, tile), tiles of a latent adjacent: the launch reads P front to back
+    const int64_t item = static_cast<int64_t>(blockIdx.x - n_long_blocks) * (blockDim.x >> 6) + wave_in_block();
+    const int64_t f = item / tps;
     if (f >= F) return;  // uniform per wavefront
+    const int t = static_cast<int>(item - f * tps);
     const uint32_t s0 = begin[f];
     const uint32_t n = begin[f + 1] - s0;
     if (n > static_cast<uint32_t>(kSegChunk)) return;
-    for (int t = 0; t < tps; ++t) {
-      const int pc = t * (kWave * VEC) + lane * VEC;
-      const int d0 = col0 + pc;
-      float acc[VEC];
+    const int pc = t * (kWave * VEC) + lane * VEC;
+    const int d0 = col0 + pc;
+    float acc[VEC];
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-      accumulate_rows<PT, VEC, U, FLEXSAE_REDUCE_NT>(P, s0, static_cast<int>(n), slice_w, pc, acc);
-      if (scale) {  // the rows were produced for a unit upstream gradient
-        const float g = scale[0];
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    accumulate_rows<PT, VEC, U, FLEXSAE_REDUCE_NT>(P, s0, static_cast<int>(n), slice_w, pc, acc);
+    if (scale) {  // the rows were produced for a unit upstream gradient
+      const float g = scale[0];
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) acc[i] *= g;
-      }
-      if (d0 < D) store_vec<GT, VEC, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
+      for (int i = 0; i < VEC; ++i) acc[i] *= g;
     }
+    if (d0 < D) store_vec<GT, VEC, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
     return;
   }
   const uint32_t n_long = *long_count;
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-    accumulate_rows<PT, VEC, U, FLEXSAE_REDUCE_NT>(P, c.s0, static_cast<int>(c.s1 - c.s0), slice_w, pc, acc);
+    accumulate_rows<PT, VEC, 8, FLEXSAE_REDUCE_NT>(P, c.s0, static_cast<int>(c.s1 - c.s0), slice_w, pc, acc);
     store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
   }
 }
