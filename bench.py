@@ -39,8 +39,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_k128", choices=sorted(WORKLOADS))
     ap.add_argument("--shape", default="", help="override B,K,F,D of the workload (tuning aid)")
-    ap.add_argument("--no-flat-mode", action="store_true",
-                    help="skip the extra timing of the hierarchical loss in flat-memory mode")
+    ap.add_argument("--no-other-mode", action="store_true",
+                    help="skip the extra timing of the hierarchical loss in its other memory mode (staged / flat)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows in the CPU-baseline sample (0 = auto)")
     return ap.parse_args()
@@ -212,15 +212,18 @@ def main():
     hier_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
     hier_peak = torch.cuda.max_memory_allocated() - base_mem
     Wp.grad = vp.grad = bp.grad = None
-    # the same step with nothing staged between forward and backward (flat memory): forward
-    # kernel + sliced backward
-    flat_ms = flat_peak = None
-    if not args.no_flat_mode:
-        stage_budget = flex.ops._hier_stage_bytes
-        flex.set_hier_stage_bytes(0)
-        torch.cuda.reset_peak_memory_stats()
-        flat_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
-        flat_peak = torch.cuda.max_memory_allocated() - base_mem
+    # the same step in the other memory mode of the API: with a stage budget that holds all per-pair
+    # contributions between forward and backward (faster, memory grows with B*K*D) when the run
+    # above kept memory flat (the default), and the other way round
+    other_ms = other_peak = None
+    main_staged = bool(flex.ops._stage_fits(idx, W)) and flex.ops._train_supported(W, K)
+    if not args.no_other_mode and flex.ops._train_supported(W, K):
+        stage_budget = flex.ops.hier_stage_bytes()
+        flex.set_hier_stage_bytes(0 if main_staged else torch.cuda.get_device_properties(dev).total_memory // 8)
+        if bool(flex.ops._stage_fits(idx, W)) != main_staged:
+            torch.cuda.reset_peak_memory_stats()
+            other_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
+            other_peak = torch.cuda.max_memory_allocated() - base_mem
         flex.set_hier_stage_bytes(stage_budget)
     Wp.grad = vp.grad = bp.grad = None
     torch.cuda.reset_peak_memory_stats()
@@ -245,10 +248,14 @@ def main():
     scratch = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
     # same decision as the API: the fused training step runs when the stage budget holds every
     # per-pair contribution at once (one slice as wide as D); otherwise forward + sliced backward
+    # (staged); failing that, the same kernel slice by slice with an immediate reduction (sliced);
+    # shapes the training-step kernel does not cover run forward + sliced backward (unfused)
     fused = (os.environ.get("FLEXSAE_FUSED_TRAINING", "1") not in ("", "0") and scratch > 0
-             and flex.ops._stage_fits(idx, W) and flex.ops._train_supported(W, K)
+             and flex.ops._train_supported(W, K)
              and bool(lib.flexsae_hier_fwd_bwd_supported(ctypes.byref(sh))))
-    slice_cols = D if fused else max(1, scratch // (B * K * p_size))
+    staged = fused and flex.ops._stage_fits(idx, W)
+    hier_mode = "staged" if staged else "sliced" if fused else "unfused"
+    slice_cols = D if staged else max(1, scratch // (B * K * p_size))
     bws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
     bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
     tile = 64 * (4 if D % 4 == 0 else 2 if D % 2 == 0 else 1)
@@ -265,7 +272,7 @@ def main():
                                         p(dvals), p(dbias), p(bws), bws_bytes, flags, None, st()),
                    "flexsae_hier_bwd")
 
-    PRE, REUSE, SWEEP, REDUCE = 1, 2, 4, 8
+    PRE, REUSE, SWEEP, REDUCE, NO_DW = 1, 2, 4, 8, 32
     fwd_k_ms = time_kernel_events(torch, lambda: None, fwd_launch, args.steps, args.warmup)
     step_entry_ms = None
     if fused:
@@ -276,7 +283,9 @@ def main():
                                                 st()), "flexsae_hier_fwd_bwd")
 
         step_entry_ms = time_kernel_events(torch, lambda: None, train_launch, args.steps, args.warmup)
-        sweep_ms = time_kernel_events(torch, lambda: None, lambda: train_launch(PRE | REUSE | SWEEP), args.steps, 1)
+        # the training-step kernel(s) alone: deferred reduction when staged, no dW when sliced
+        sweep_ms = time_kernel_events(torch, lambda: None,
+                                      lambda: train_launch(PRE | REUSE | (SWEEP if staged else NO_DW)), args.steps, 1)
         reduce_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(PRE | REUSE | REDUCE), args.steps, 1)
         bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
         sweep_name = "hier_train_kernel"
@@ -316,7 +325,7 @@ def main():
     traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file) and not args.shape:
         with open(traffic_file) as fh:
-            rec = json.load(fh).get(f"{args.workload}:{'fused' if fused else scratch >> 20}")
+            rec = json.load(fh).get(f"{args.workload}:{'fused' if staged else scratch >> 20}")
         if rec:
             traffic = rec.get(f"{sweep_name}_bytes_per_launch")
     roofline = {
@@ -347,7 +356,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
                                f"indices {dist}", "B": B, "K": K, "F": F, "D": D,
-                   "hier_scratch_mb": scratch >> 20, "fused_training_step": bool(fused),
+                   "hier_scratch_mb": scratch >> 20, "fused_training_step": bool(fused), "hier_mode": hier_mode,
                    "hier_stage_mb": flex.ops.hier_stage_bytes(dev) >> 20},
         "roofline": roofline,
         "step_hbm": {"algorithmic_bytes": abytes["hier_step"],
@@ -369,9 +378,9 @@ def main():
         "topk": {"ms_per_step": round(topk_ms, 4), "algorithmic_bytes": abytes["topk_step"],
                  "achieved_GBps": round(gbps(abytes["topk_step"], topk_ms), 1)},
         "hier_over_topk_latency": round(hier_ms / topk_ms, 3),
-        "hier_flat_memory_mode": None if flat_ms is None else {
-            "ms_per_step": round(flat_ms, 4), "over_topk_latency": round(flat_ms / topk_ms, 3),
-            "peak_mem_gib": round(flat_peak / 2 ** 30, 3)},
+        ("hier_flat_memory_mode" if main_staged else "hier_staged_mode"): None if other_ms is None else {
+            "ms_per_step": round(other_ms, 4), "over_topk_latency": round(other_ms / topk_ms, 3),
+            "peak_mem_gib": round(other_peak / 2 ** 30, 3)},
         "peak_mem_gib": {"hier": round(hier_peak / 2 ** 30, 3), "topk": round(topk_peak / 2 ** 30, 3),
                          "inputs": round(base_mem / 2 ** 30, 3)},
     }

@@ -29,6 +29,7 @@ BWD_REUSE_PAIR_LIST = 2
 BWD_SWEEP_ONLY = 4
 BWD_REDUCE_ONLY = 8
 BWD_SCALE_BY_GRAD_OUT = 16
+BWD_NO_DW = 32
 
 
 class Shape(ctypes.Structure):

@@ -401,7 +401,11 @@ void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int6
                          int64_t cols, int col0, int slice_w, hipStream_t st) {
   const int64_t n_items = s->B * (cols / 128);
   // K == KMAX (the usual powers of two) runs the variant without per-step bound tests
-  const auto kernel = s->K == KMAX ? hier_train_kernel<WT, PT, KMAX, true> : hier_train_kernel<WT, PT, KMAX, false>;
+  const bool stream = slice_w >= d_pad;  // all of P in one launch: streaming stores
+  const auto kernel = s->K == KMAX
+                          ? (stream ? hier_train_kernel<WT, PT, KMAX, true, true> : hier_train_kernel<WT, PT, KMAX, true, false>)
+                          : (stream ? hier_train_kernel<WT, PT, KMAX, false, true>
+                                    : hier_train_kernel<WT, PT, KMAX, false, false>);
   hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
                      indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
                      coef, slot, P, dvals, s_final, d_pad, loss_partial, status_flag, n_items, s->B, col0,
@@ -856,16 +860,17 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
                          size_t workspace_bytes, int flags, int *status_flag, void *stream) {
   int rc = check_shape(s);
   if (rc != FLEXSAE_OK) return rc;
-  const bool defer_reduce = (flags & FLEXSAE_BWD_SWEEP_ONLY) != 0;
+  const bool no_dw = (flags & FLEXSAE_BWD_NO_DW) != 0;
+  const bool defer_reduce = (flags & FLEXSAE_BWD_SWEEP_ONLY) != 0 && !no_dw;
   if (!indices || !weight || !vals || !bias || !target || !loss || !dvals || !dbias ||
-      (!defer_reduce && (!dW || !valid_dtype(dW_dtype))))
+      (!defer_reduce && !no_dw && (!dW || !valid_dtype(dW_dtype))))
     return FLEXSAE_ERR_INVALID_ARGUMENT;
   if (!train_supported(s)) return FLEXSAE_ERR_UNSUPPORTED;
   const HierBwdPlan pl = plan_hier_bwd(s);  // D % 4 == 0 here, so tiles are 256 columns
   if (!aligned(indices, 8) || !aligned(weight, 4 * dtype_size(s->weight_dtype)) ||
       !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(bias, 2 * dtype_size(s->bias_dtype)) ||
       !aligned(target, 2 * dtype_size(s->target_dtype)) || !aligned(loss, 4) ||
-      (!defer_reduce && !aligned(dW, 4 * dtype_size(dW_dtype))) || !aligned(dvals, 16) ||
+      (!defer_reduce && !no_dw && !aligned(dW, 4 * dtype_size(dW_dtype))) || !aligned(dvals, 16) ||
       !aligned(dbias, 16))
     return FLEXSAE_ERR_ALIGNMENT;
   if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, pl.tile))
@@ -888,9 +893,11 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   const double count = static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D);
   const float coef = static_cast<float>(2.0 / count);
   const TrainArgs ta = {bias, target};
-  launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, nullptr, coef, dW, dW_dtype, dvals,
-                          dbias, ws, flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY), status_flag,
-                          st, &ta);
+  // without dW the reductions are left out like in the deferred case (dW_dtype only selects a template then)
+  launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, nullptr, coef, dW,
+                          no_dw ? s->weight_dtype : dW_dtype, dvals, dbias, ws,
+                          (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY)) | (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0),
+                          status_flag, st, &ta);
   rc = launch_status();
   if (rc != FLEXSAE_OK) return rc;
   hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(1024), 0, st,

@@ -3,10 +3,6 @@
 
 #include "common.hpp"
 
-#ifndef FLEXSAE_TRAIN_NT
-#define FLEXSAE_TRAIN_NT true
-#endif
-
 namespace flexsae {
 
 // A gathered piece of a weight row (two consecutive columns) kept in raw form.
@@ -56,7 +52,11 @@ struct RowPiece2<f16_t> {
 // Row gathers and contribution stores go through per-row buffer descriptors: their address
 // arithmetic runs on the scalar unit, lanes beyond column D read zeros (so their dot products
 // vanish), and what such lanes store lands in the padding columns of P, which nobody reads.
-template <typename WT, typename PT, int KMAX, bool FULL>
+// STREAM: the contributions are stored with the non-temporal hint.  That is the faster choice
+// when all of P is written before any of it is read back (it is far larger than the caches);
+// when P is one slice that the reduction reads right after this launch, plain stores leave part
+// of it in the memory-side cache and the pair of launches is faster.
+template <typename WT, typename PT, int KMAX, bool FULL, bool STREAM>
 __global__ __launch_bounds__(256) void hier_train_kernel(
     const int64_t *__restrict__ indices, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
             packed[0] = __float_as_uint(contrib[0]);
             packed[1] = __float_as_uint(contrib[1]);
           }
-          descriptor_store<sizeof(packed), FLEXSAE_TRAIN_NT>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
+          descriptor_store<sizeof(packed), STREAM>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
           dots[u] = dot;  // zero where the lane is beyond column D: its w is zero
         }
       }
@@ -216,12 +216,14 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   store_vec<float, VEC>(s_final, b * s_final_ld + col0 + pc, S);
 }
 
-// dst[i] = src[i] * scale[0] (dtype in, same dtype out); used to apply the upstream gradient to
-// the unit-gradient results of the training-step kernel.
+// dst[i] = src[i] * scale[0] (dtype in, same dtype out; dst may be src); used to apply the
+// upstream gradient to the unit-gradient results of the training-step kernel.  In place with a
+// scale of exactly one, the usual loss.backward(), the kernel returns at once.
 template <typename T>
-__global__ void scale_kernel(void *__restrict__ dst, const void *__restrict__ src, int64_t n,
+__global__ void scale_kernel(void *dst, const void *src, int64_t n,
                              const float *__restrict__ scale) {
   const float g = scale[0];
+  if (dst == src && g == 1.0f) return;  // in place by one: nothing to do
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t n4 = n >> 2;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) {

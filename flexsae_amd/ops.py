@@ -173,31 +173,26 @@ def set_hier_scratch_bytes(nbytes: int) -> None:
 
 
 # Memory the fused training step may hold between forward and backward: all B*K*D per-pair
-# contributions (2 bytes each for bf16 weights, else 4) plus the pair list.  Unless set, the
-# budget is one eighth of the device's memory (36 GB on a 288 GB MI355X).
-_hier_stage_bytes = (int(os.environ["FLEXSAE_HIER_STAGE_MB"]) << 20) if "FLEXSAE_HIER_STAGE_MB" in os.environ else None
-_device_stage_default = {}
+# contributions (2 bytes each for bf16 weights, else 4) plus the pair list.  The default is 0:
+# memory stays flat (the step runs slice by slice inside the scratch above, and only the weight
+# gradient itself waits for the backward).  A budget that covers the contributions makes the step
+# about 5 % faster at the price of that memory.
+_hier_stage_bytes = (int(os.environ["FLEXSAE_HIER_STAGE_MB"]) << 20) if "FLEXSAE_HIER_STAGE_MB" in os.environ else 0
 
 
 def set_hier_stage_bytes(nbytes) -> None:
-    """Upper bound (bytes) on what the fused training step keeps alive from forward to backward.
-    Calls whose contributions do not fit run the separate forward and sliced backward instead;
-    0 switches the fused step off for every shape (flat memory); None restores the default, one
-    eighth of the device's memory."""
+    """Upper bound (bytes) on what the fused training step may keep alive from forward to
+    backward beyond the gradients themselves.  0 or None (the default): nothing, the step runs
+    slice by slice in the scratch of ``set_hier_scratch_bytes`` and memory stays flat.  A budget
+    that holds all B*K*D per-pair contributions (2 bytes each for bf16 weights, else 4) lets the
+    step write them once and reduce them in the backward, which is a little faster."""
     global _hier_stage_bytes
-    _hier_stage_bytes = None if nbytes is None else int(nbytes)
+    _hier_stage_bytes = 0 if nbytes is None else int(nbytes)
 
 
-def hier_stage_bytes(device) -> int:
-    """The stage budget in force for tensors on ``device``."""
-    if _hier_stage_bytes is not None:
-        return _hier_stage_bytes
-    index = torch.device(device).index
-    if index is None:
-        index = torch.cuda.current_device()
-    if index not in _device_stage_default:
-        _device_stage_default[index] = torch.cuda.get_device_properties(index).total_memory // 8
-    return _device_stage_default[index]
+def hier_stage_bytes(device=None) -> int:
+    """The stage budget in force (the same for every device)."""
+    return _hier_stage_bytes
 
 
 # ---- one pair list for both losses ---------------------------------------------------------
@@ -368,12 +363,13 @@ _fused_training = os.environ.get("FLEXSAE_FUSED_TRAINING", "1") not in ("", "0")
 def set_fused_training(enabled: bool) -> None:
     """Enable/disable the fused forward + reverse walk of the hierarchical loss (default on).
 
-    It is used when gradients are required AND the stage budget (``set_hier_stage_bytes``)
-    can hold all per-pair contributions at once (B*K*D elements): the weight rows are then
-    gathered once per training step instead of twice, the contributions wait in the scratch and
-    the backward only runs the segment reduction, scaled by the upstream gradient.  Code that
-    evaluates the loss with gradients enabled but never calls ``backward()`` pays for the reverse
-    walk anyway: switch it off there or use ``torch.no_grad()``."""
+    When gradients are required, loss and gradients come out of one pass that gathers the weight
+    rows once per training step instead of twice; the gradients are those of a unit upstream
+    gradient and the backward only scales them.  By default the pass runs slice by slice with an
+    immediate segment reduction (flat memory); with a stage budget (``set_hier_stage_bytes``)
+    that holds all per-pair contributions, they are written once and reduced in the backward.
+    Code that evaluates the loss with gradients enabled but never calls ``backward()`` pays for
+    the reverse walk anyway: switch it off there or use ``torch.no_grad()``."""
     global _fused_training
     _fused_training = bool(enabled)
 
@@ -384,8 +380,8 @@ def _train_supported(weight: Tensor, K: int) -> bool:
 
 
 def _stage_fits(indices: Tensor, weight: Tensor) -> bool:
-    """The fused pass keeps one contribution per (b, k, d) alive until the backward; it is taken
-    only when the stage budget covers that."""
+    """Staging keeps one contribution per (b, k, d) alive until the backward; it is chosen only
+    when the stage budget covers that."""
     B, K = indices.shape
     D = weight.shape[1]
     p_size = 2 if weight.dtype == torch.bfloat16 else 4
@@ -488,6 +484,136 @@ def _train_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_stage):
 hier_train.register_autograd(_train_backward, setup_context=_train_setup_context)
 
 
+@torch.library.custom_op("flexsae_amd::hier_train_sliced", mutates_args=())
+def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
+                      target: Tensor) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Fused forward + reverse walk in column slices, each reduced right away (flat memory).
+
+    Used when the contributions of a whole step do not fit the stage budget: the scratch is one
+    slice of them (``set_hier_scratch_bytes``), and every slice gathers its weight-row pieces once
+    for both walks.  Returns (loss, dvals, dbias, dW), the gradients for a unit upstream gradient;
+    the backward scales them."""
+    B, K, F, D = _validate(indices, weight, vals, bias, target)
+    lib = _lib.load()
+    indices, weight, vals, bias, target = (t.contiguous() for t in (indices, weight, vals, bias, target))
+    dev = weight.device
+    with torch.cuda.device(dev):
+        shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
+        p_size = 2 if weight.dtype == torch.bfloat16 else 4
+        slice_cols = max(1, _hier_scratch_bytes // (B * K * p_size))
+        ws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        dW = torch.empty_like(weight)
+        dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
+        dbias = torch.empty((D,), dtype=torch.float32, device=dev)
+        flag = _flag_for(dev)
+        cached = _pair_lookup(indices, F)
+        if cached is not None:
+            _pair_import(lib, shape, workspace, cached)
+        flags = _lib.BWD_REUSE_PAIR_LIST if cached is not None else 0
+        rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
+                                      _ptr(target), _ptr(loss), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals),
+                                      _ptr(dbias), _ptr(workspace), ws_bytes, flags, _ptr(flag), _stream())
+        _lib.check(rc, "flexsae_hier_fwd_bwd")
+        if cached is None:
+            _pair_export(lib, shape, workspace, indices, F)
+        if _check_indices:
+            check_index_flag(dev)
+    return loss, dvals, dbias, dW
+
+
+@hier_train_sliced.register_fake
+def _(indices, weight, vals, bias, target):
+    return (weight.new_empty((), dtype=torch.float32), vals.new_empty(vals.shape, dtype=torch.float32),
+            weight.new_empty((weight.shape[1],), dtype=torch.float32), torch.empty_like(weight))
+
+
+@torch.library.custom_op("flexsae_amd::scale_by", mutates_args=())
+def scale_by(x: Tensor, grad_out: Tensor) -> Tensor:
+    """x * grad_out (a 0-dim scalar on the device), in x's dtype; replaces the reference's
+    ``dW.mul_(grad)`` (hierarchical_kernels.py:294-297) after a unit-gradient pass."""
+    lib = _lib.load()
+    dev = x.device
+    with torch.cuda.device(dev):
+        g = _grad_scalar(grad_out, dev)
+        x = x.contiguous()
+        out = torch.empty_like(x)
+        rc = lib.flexsae_scale(_ptr(out), _ptr(x), _DTYPES[x.dtype], x.numel(), _ptr(g), _stream())
+        _lib.check(rc, "flexsae_scale")
+    return out
+
+
+@scale_by.register_fake
+def _(x, grad_out):
+    return torch.empty_like(x)
+
+
+@torch.library.custom_op("flexsae_amd::scale_", mutates_args=("x",))
+def scale_(x: Tensor, grad_out: Tensor) -> None:
+    """x *= grad_out in place (x contiguous); a grad_out of exactly one costs an empty launch."""
+    lib = _lib.load()
+    dev = x.device
+    if not x.is_contiguous():
+        raise ValueError("scale_ needs a contiguous tensor")
+    with torch.cuda.device(dev):
+        g = _grad_scalar(grad_out, dev)
+        rc = lib.flexsae_scale(_ptr(x), _ptr(x), _DTYPES[x.dtype], x.numel(), _ptr(g), _stream())
+        _lib.check(rc, "flexsae_scale")
+
+
+@scale_.register_fake
+def _(x, grad_out):
+    return None
+
+
+def _is_traced(t: Tensor) -> bool:
+    """True while a compiler traces the call (fake or functional tensors instead of real ones)."""
+    return type(t) is not torch.Tensor or torch.compiler.is_compiling()
+
+
+def _train_sliced_setup_context(ctx, inputs, output):
+    indices, weight, vals, bias, target = inputs
+    _, dvals, dbias, dW = output
+    ctx.mark_non_differentiable(dvals, dbias, dW)
+    ctx.leaf_dtypes = (vals.dtype, bias.dtype)
+    ctx.set_materialize_grads(False)
+    # The unit-gradient dW is as large as the weight.  In eager mode it is kept outside the saved
+    # tensors so that the backward can scale it in place and hand the very buffer on as the weight
+    # gradient (it carries no autograd history, so keeping it on ctx forms no reference cycle).
+    ctx.dw_in_place = not _is_traced(dW)
+    if ctx.dw_in_place:
+        ctx.save_for_backward(indices, weight, vals, bias, target, dvals, dbias)
+        ctx.dw_unit = dW if ctx.needs_input_grad[1] else None
+    else:
+        ctx.save_for_backward(indices, weight, vals, bias, target, dvals, dbias, dW)
+
+
+def _train_sliced_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_dw):
+    if grad_loss is None:
+        return None, None, None, None, None
+    g = grad_loss.to(torch.float32)
+    vdt, bdt = ctx.leaf_dtypes
+    if not ctx.dw_in_place:
+        indices, weight, vals, bias, target, dvals, dbias, dW_unit = ctx.saved_tensors
+        dW = scale_by(dW_unit, g) if ctx.needs_input_grad[1] else None
+    else:
+        indices, weight, vals, bias, target, dvals, dbias = ctx.saved_tensors
+        dW = None
+        if ctx.needs_input_grad[1]:
+            dW = ctx.dw_unit
+            ctx.dw_unit = None  # the buffer now belongs to whoever receives the gradient
+            if dW is None:
+                # a second backward through a retained graph: the buffer went with the first one
+                with torch.no_grad():
+                    _, dvals, dbias, dW = hier_train_sliced(indices, weight, vals, bias, target)
+            scale_(dW, g)
+    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None
+
+
+hier_train_sliced.register_autograd(_train_sliced_backward, setup_context=_train_sliced_setup_context)
+
+
 def _hier_backward(ctx, grad_loss, grad_resid):
     indices, weight, vals, resid = ctx.saved_tensors
     if grad_loss is None:
@@ -526,8 +652,11 @@ def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, 
         indices = indices.to(torch.int64)
     needs_grad = torch.is_grad_enabled() and (weight.requires_grad or vals.requires_grad or bias.requires_grad)
     if (needs_grad and _fused_training and weight.dim() == 2 and indices.dim() == 2
-            and _train_supported(weight, indices.shape[1]) and _stage_fits(indices, weight)):
-        return hier_train(indices, weight, vals, bias, target)[0]
+            and _train_supported(weight, indices.shape[1])):
+        if _stage_fits(indices, weight):
+            return hier_train(indices, weight, vals, bias, target)[0]
+        if _hier_scratch_bytes > 0:
+            return hier_train_sliced(indices, weight, vals, bias, target)[0]
     return hier_fwd(indices, weight, vals, bias, target)[0]
 
 

@@ -63,8 +63,11 @@ enum {
                                      /* already in the workspace; with REUSE_PAIR_LIST and a    */
                                      /* single-slice workspace only grad_out, dW and workspace  */
                                      /* are read (the rest may be NULL): the deferred reduction */
-  FLEXSAE_BWD_SCALE_BY_GRAD_OUT = 16 /* deferred reduction only: the contributions were made    */
+  FLEXSAE_BWD_SCALE_BY_GRAD_OUT = 16,/* deferred reduction only: the contributions were made    */
                                      /* for a unit upstream gradient; multiply dW by grad_out[0]*/
+  FLEXSAE_BWD_NO_DW = 32             /* flexsae_hier_fwd_bwd only: dW is not wanted (may be     */
+                                     /* NULL); the segment reductions are left out, whatever    */
+                                     /* the width of the workspace, and nothing is deferred     */
 };
 
 /* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^29; B*K < 2^32. */
@@ -164,7 +167,8 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, con
                          size_t workspace_bytes, int flags, int *status_flag, void *stream);
 
 /*
- * dst[n] = src[n] * scale[0]  (same dtype in and out; `scale` is a device fp32 scalar).
+ * dst[n] = src[n] * scale[0]  (same dtype in and out; `scale` is a device fp32 scalar).  dst may
+ * be src (in place); then a scale of exactly 1 costs one empty launch.
  * replaces: the dW.mul_(grad) pass of HierarchicalSAELossFunction.backward
  *           (hierarchical_kernels.py:294-297), needed only after flexsae_hier_fwd_bwd.
  */

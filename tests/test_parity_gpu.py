@@ -31,6 +31,9 @@ def _announce(*what):
     print("[case]", *what, flush=True)
 
 
+STAGE_ALL = 1 << 40  # a stage budget that holds the contributions of every test shape
+
+
 def _run_op(mode, args_cpu, grad_out):
     idx, W, v, b, t = _to_dev(args_cpu)
     W.requires_grad_()
@@ -65,15 +68,20 @@ def _check_against_oracle(mode, args_cpu, dtype, grad_out, got, ref_tols=True):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
 @pytest.mark.parametrize("B,K,F,D", PARAMS)
-@pytest.mark.parametrize("mode", ["hier", "topk"])
+@pytest.mark.parametrize("mode", ["hier", "hier_staged", "topk"])
 def test_reference_matrix(mode, B, K, F, D, dtype):
     """The reference's 26 shapes x 3 dtypes x 2 losses, with a random scalar upstream gradient
-    (reference tests/test_all_kernels.py:20-66)."""
+    (reference tests/test_all_kernels.py:20-66).  The hierarchical loss runs in both memory modes:
+    flat (the default: training step slice by slice) and with all contributions staged."""
     _announce("matrix", mode, B, K, F, D, dtype)
     args = make_inputs(B, K, F, D, dtype=dtype)
     grad_out = float(torch.randn((), generator=torch.Generator().manual_seed(B * K + D)))
-    got = _run_op(mode, args, grad_out)
-    _check_against_oracle(mode, args, dtype, grad_out, got)
+    flex.set_hier_stage_bytes(STAGE_ALL if mode == "hier_staged" else None)
+    try:
+        got = _run_op(mode.split("_")[0], args, grad_out)
+    finally:
+        flex.set_hier_stage_bytes(None)
+    _check_against_oracle(mode.split("_")[0], args, dtype, grad_out, got)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
@@ -136,16 +144,21 @@ def test_training_step_unsupported_shapes_and_scale():
         assert rc == 0 and torch.equal(y, (x.float() * -2.5).to(dt))
 
 
-def test_fused_training_backward_twice_and_no_grad():
+@pytest.mark.parametrize("stage", [STAGE_ALL, None], ids=["staged", "sliced"])
+def test_fused_training_backward_twice_and_no_grad(stage):
     """retain_graph + two backward calls accumulate correctly; no_grad / non-leaf-free inputs take
     the forward-only kernel."""
     args = make_inputs(32, 16, 100, 512, dtype=torch.bfloat16, seed=8)
     idx, W, v, b, t = _to_dev(args)
     W.requires_grad_()
-    loss = flex.triton_hierarchical_sae_loss(idx, W, v, b, t)
-    loss.backward(torch.tensor(2.0, device=DEV), retain_graph=True)
-    g1 = W.grad.clone()
-    loss.backward(torch.tensor(-0.5, device=DEV))
+    flex.set_hier_stage_bytes(stage)
+    try:
+        loss = flex.triton_hierarchical_sae_loss(idx, W, v, b, t)
+        loss.backward(torch.tensor(2.0, device=DEV), retain_graph=True)
+        g1 = W.grad.clone()
+        loss.backward(torch.tensor(-0.5, device=DEV))
+    finally:
+        flex.set_hier_stage_bytes(None)
     L, rW, _, _ = oracle.loss_grads(oracle.HIER, *args, grad_out=1.5)
     assert rel_err(W.grad.float().cpu(), rW) < 2e-2
     assert rel_err(g1.float().cpu(), rW * (2.0 / 1.5)) < 1e-2
@@ -368,18 +381,28 @@ def test_hier_gradients_are_reproducible_bit_for_bit(dtype):
         assert torch.equal(a, c)
 
 
-@pytest.mark.parametrize("mode", ["segment", "atomic"])
+@pytest.mark.parametrize("mode", ["sliced", "segment", "atomic"])
 def test_hier_backward_variants_through_the_op(mode):
-    """Both stand-alone backward implementations behind the public op (scratch budget 0 = atomic
-    fallback, 1 MiB = several slices), reached because the stage budget is too small to fuse."""
+    """What the public op runs when the stage budget is too small to keep a whole step's
+    contributions: the training-step kernel slice by slice (1 MiB of scratch = several slices);
+    with the fusion switched off, forward + sliced segment backward; with a scratch budget of 0,
+    forward + the atomic fallback."""
     args = make_inputs(48, 32, 200, 768, dtype=torch.bfloat16, seed=13)
     flex.set_hier_scratch_bytes(0 if mode == "atomic" else 1 << 20)
     flex.set_hier_stage_bytes(1 << 20)
+    flex.set_fused_training(mode != "segment")
     try:
         got = _run_op("hier", args, 1.5)
+        if mode == "sliced":  # upstream gradient 1: bit-identical to the staged step
+            one = _run_op("hier", args, 1.0)
+            flex.set_hier_stage_bytes(STAGE_ALL)
+            staged = _run_op("hier", args, 1.0)
+            for a, c in zip(one, staged):
+                assert torch.equal(a, c)
     finally:
         flex.set_hier_scratch_bytes(256 << 20)
         flex.set_hier_stage_bytes(None)
+        flex.set_fused_training(True)
     _check_against_oracle("hier", args, torch.bfloat16, 1.5, got)
 
 
@@ -461,8 +484,8 @@ def test_opcheck_and_compile(mode):
     W.requires_grad_()
     v.requires_grad_()
     b.requires_grad_()
-    ops_ = ([torch.ops.flexsae_amd.hier_fwd, torch.ops.flexsae_amd.hier_train] if mode == "hier"
-            else [torch.ops.flexsae_amd.topk_fwd])
+    ops_ = ([torch.ops.flexsae_amd.hier_fwd, torch.ops.flexsae_amd.hier_train,
+             torch.ops.flexsae_amd.hier_train_sliced] if mode == "hier" else [torch.ops.flexsae_amd.topk_fwd])
     for op in ops_:
         torch.library.opcheck(op, (idx, W, v, b, t),
                               test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
@@ -471,17 +494,29 @@ def test_opcheck_and_compile(mode):
     assert abs(compiled.item() - 2.0 * eager.item()) <= 1e-6 * abs(eager.item())
     compiled.backward()
     assert W.grad is not None and v.grad is not None and b.grad is not None
+    if mode == "hier":  # the same with the contributions staged between forward and backward
+        want = W.grad.clone()
+        W.grad = None
+        flex.set_hier_stage_bytes(STAGE_ALL)
+        try:
+            sliced = torch.compile(lambda *a: FUSED[mode](*a) * 2.0, fullgraph=True, backend="aot_eager")(idx, W, v, b, t)
+            sliced.backward()
+        finally:
+            flex.set_hier_stage_bytes(None)
+        assert abs(sliced.item() - compiled.item()) <= 1e-6 * abs(compiled.item())
+        assert rel_err(W.grad.cpu(), want.cpu().numpy()) < 1e-5
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("order", ["topk_first", "hier_first"])
-@pytest.mark.parametrize("fused", [True, False], ids=["fused", "unfused"])
+@pytest.mark.parametrize("fused", ["sliced", "staged", "unfused"])
 def test_shared_pair_list_changes_nothing(order, fused, dtype):
     """Inside shared_pair_list() the second loss on the same indices reuses the first one's pair
     list; loss and gradients stay bit-identical to the unshared calls."""
     args = make_inputs(64, 16, 300, 512, dtype=dtype, seed=77)
     modes = ["topk", "hier"] if order == "topk_first" else ["hier", "topk"]
-    flex.set_fused_training(fused)
+    flex.set_fused_training(fused != "unfused")
+    flex.set_hier_stage_bytes(STAGE_ALL if fused == "staged" else None)
     try:
         plain = {m: _run_op(m, args, 0.8) for m in modes}
         shared = {}
@@ -496,6 +531,7 @@ def test_shared_pair_list_changes_nothing(order, fused, dtype):
         assert flex.ops._pair_cache is None
     finally:
         flex.set_fused_training(True)
+        flex.set_hier_stage_bytes(None)
     torch.cuda.synchronize()
     for m in modes:
         for a, c in zip(plain[m], shared[m]):
@@ -562,12 +598,16 @@ def test_random_shapes(seed):
     grad_out = float(rng.normal())
     _announce("random", seed, (B, K, F, D), dtype, grad_out)
     args = make_inputs(B, K, F, D, dtype=dtype, seed=seed)
-    for mode in ("hier", "topk"):
-        got = _run_op(mode, args, grad_out)
-        _check_against_oracle(mode, args, dtype, grad_out, got, ref_tols=False)
+    flex.set_hier_stage_bytes(STAGE_ALL if seed % 2 else None)  # odd seeds: contributions staged
+    try:
+        for mode in ("hier", "topk"):
+            got = _run_op(mode, args, grad_out)
+            _check_against_oracle(mode, args, dtype, grad_out, got, ref_tols=False)
+    finally:
+        flex.set_hier_stage_bytes(None)
 
 
-@pytest.mark.parametrize("mode", ["hier", "topk"])
+@pytest.mark.parametrize("mode", ["hier", "hier_staged", "topk"])
 def test_step_can_be_captured_in_a_graph(mode):
     """Forward + backward recorded into a HIP graph (no memset nodes, no synchronisation, no
     allocation outside torch's graph pool) and replayed with new input values, with eager work
@@ -577,8 +617,16 @@ def test_step_can_be_captured_in_a_graph(mode):
     W.requires_grad_()
     v.requires_grad_()
     b.requires_grad_()
-    fn = FUSED[mode]
+    loss_name = mode.split("_")[0]
+    fn = FUSED[loss_name]
+    flex.set_hier_stage_bytes(STAGE_ALL if mode == "hier_staged" else None)
+    try:
+        _graph_capture_body(loss_name, fn, idx, W, v, b, t)
+    finally:
+        flex.set_hier_stage_bytes(None)
 
+
+def _graph_capture_body(mode, fn, idx, W, v, b, t):
     def step():
         W.grad = v.grad = b.grad = None
         loss = fn(idx, W, v, b, t)
