@@ -912,7 +912,7 @@ int flexsae_scale(void *dst, const void *src, int dtype, int64_t n, const float 
   if (!aligned(src, 4 * dtype_size(dtype)) || !aligned(dst, 4 * dtype_size(dtype)) || !aligned(scale, 4))
     return FLEXSAE_ERR_ALIGNMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(grid_for(ceil_div(n, 4), 256, 1 << 16));
+  const dim3 grid(grid_for(ceil_div(n, 4), 256, 4096));  // few blocks: in place by one they all return at once
   switch (dtype) {
     case FLEXSAE_F32:
       hipLaunchKernelGGL(scale_kernel<float>, grid, dim3(256), 0, st, dst, src, n, scale);

@@ -58,7 +58,7 @@ def hier_backward(indices, weight, vals, resid, grad_out, flag=None, slice_cols=
     return rc, dW, dv, db
 
 
-def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_dtype=torch.float32):
+def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_dtype=torch.float32, flags=0):
     """Fused forward+backward for a unit upstream gradient -> (rc, loss, dW, dvals, dbias)."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
@@ -70,14 +70,14 @@ def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_
     nbytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
     ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
     rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(bias), ptr(target),
-                                  ptr(loss), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, 0,
+                                  ptr(loss), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, flags,
                                   ptr(flag), stream())
     return rc, loss, dW, dv, db
 
 
-def scale(src, g):
+def scale(src, g, in_place=False):
     lib = _lib.load()
-    dst = torch.full_like(src, float("nan"))
+    dst = src if in_place else torch.full_like(src, float("nan"))
     gt = torch.tensor([g], dtype=torch.float32, device=src.device)
     rc = lib.flexsae_scale(ptr(dst), ptr(src), DT[src.dtype], src.numel(), ptr(gt), stream())
     return rc, dst

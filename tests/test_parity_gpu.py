@@ -142,6 +142,23 @@ def test_training_step_unsupported_shapes_and_scale():
         x = torch.randn(1003, device=DEV).to(dt)
         rc, y = abi.scale(x, -2.5)
         assert rc == 0 and torch.equal(y, (x.float() * -2.5).to(dt))
+        for g in (1.0, 0.75):  # in place; by one the kernel leaves everything as it is
+            z = x.clone()
+            rc, z2 = abi.scale(z, g, in_place=True)
+            assert rc == 0 and z2 is z and torch.equal(z, (x.float() * g).to(dt))
+
+
+def test_training_step_without_dw():
+    """FLEXSAE_BWD_NO_DW: loss, dvals and dbias as usual, for any workspace width; dW is not touched."""
+    args = make_inputs(40, 32, 300, 1024, dtype=torch.bfloat16, seed=19)
+    idx, W, v, b, t = _to_dev(args)
+    rc, loss, dW, dv, db = abi.hier_train(idx, W, v, b, t, dw_dtype=torch.bfloat16)
+    assert rc == 0
+    for cols in (0, 256, 1 << 20):
+        rc2, loss2, dW2, dv2, db2 = abi.hier_train(idx, W, v, b, t, slice_cols=cols, dw_dtype=torch.bfloat16, flags=32)
+        torch.cuda.synchronize()
+        assert rc2 == 0 and torch.equal(loss, loss2) and torch.equal(dv, dv2) and torch.equal(db, db2)
+        assert torch.isnan(dW2.float()).all()
 
 
 @pytest.mark.parametrize("stage", [STAGE_ALL, None], ids=["staged", "sliced"])
