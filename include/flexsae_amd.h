@@ -159,6 +159,8 @@ int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const v
  * FLEXSAE_BWD_REUSE_PAIR_LIST | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SCALE_BY_GRAD_OUT finishes dW
  * with the upstream gradient folded in, so no separate scaling pass over dW is needed.  The
  * price is that the workspace (B*K*D contributions) must stay alive in between.
+ * With FLEXSAE_BWD_NO_DW (a decoder whose weight needs no gradient) the reductions are left out
+ * for any workspace width: loss, dvals and dbias as usual, dW untouched (may be NULL).
  */
 int flexsae_hier_fwd_bwd_supported(const flexsae_shape *shape);
 int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
