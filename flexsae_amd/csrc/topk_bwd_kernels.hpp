@@ -8,6 +8,10 @@
 #ifndef FLEXSAE_TOPK_ONE_GROUP
 #define FLEXSAE_TOPK_ONE_GROUP 1
 #endif
+// rows of a group of eight that share one uniform "are there rows left" test
+#ifndef FLEXSAE_TOPK_ROWS_PER_TEST
+#define FLEXSAE_TOPK_ROWS_PER_TEST 2
+#endif
 #ifndef FLEXSAE_TOPK_NT
 #define FLEXSAE_TOPK_NT true
 #endif
@@ -80,10 +84,11 @@ __device__ __forceinline__ void topk_accumulate_slots(
 // One short latent (1 to kSegChunk pairs) for one tile: the pair records of the latent are one
 // contiguous load, the residual rows are gathered through a buffer descriptor (no vector ALU work
 // for addresses) eight at a time (with the next eight already requested when registers allow),
-// and each group of eight shares one transposed wave reduction for the dvals dot products.  Groups are always
-// processed in full: slots past the end re-read the last row (a cache hit) with a val of zero,
-// which keeps the inner code free of branches.  With bf16 weights and a bf16 residual copy the
-// products run on packed pairs (dot2) without unpacking.
+// and each group of eight shares one transposed wave reduction for the dvals dot products.  Inside a
+// group, rows are requested and consumed two at a time under one uniform test, so a latent with
+// nine pairs costs ten rows, not sixteen (a test per row costs more than it saves; the odd slot
+// past the end re-reads the last row, a cache hit, with a val of zero).  With bf16 weights and a
+// bf16 residual copy the products run on packed pairs (dot2) without unpacking.
 template <typename WT, typename GT, typename RT, int VEC>
 __device__ __forceinline__ void topk_short_latent(
     const vec_t<uint32_t, 2> *__restrict__ slot_bv, const void *__restrict__ weight, int vals_dtype,
@@ -108,9 +113,14 @@ __device__ __forceinline__ void topk_short_latent(
   raw_vec_t<RT, VEC> buf_a[8], buf_b[kTwoGroups ? 8 : 1];
   auto issue = [&](raw_vec_t<RT, VEC>(&buf)[8], int j) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int jj = (j + u) < n ? (j + u) : (n - 1);
-      buf[u] = gather_raw<RT, VEC>(rows_src, lane_off, static_cast<uint32_t>(bcast_i32(my_b, jj)) * row_stride);
+    for (int h = 0; h < 8; h += FLEXSAE_TOPK_ROWS_PER_TEST) {
+      if (h == 0 || j + h < n) {  // uniform: the second half of a group only when it has rows
+#pragma unroll
+        for (int u = h; u < h + FLEXSAE_TOPK_ROWS_PER_TEST; ++u) {
+          const int jj = (j + u) < n ? (j + u) : (n - 1);
+          buf[u] = gather_raw<RT, VEC>(rows_src, lane_off, static_cast<uint32_t>(bcast_i32(my_b, jj)) * row_stride);
+        }
+      }
     }
   };
   issue(buf_a, 0);
@@ -137,40 +147,46 @@ __device__ __forceinline__ void topk_short_latent(
   auto consume = [&](const raw_vec_t<RT, VEC>(&rows)[8], int j) {  // slots j .. j+7 of the latent
     float dots[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      float dot = 0.f;
-      if constexpr (kDot2) {
-        uint32_t xw[VEC / 2];
-        __builtin_memcpy(xw, &rows[u], sizeof(xw));
+    for (int u = 0; u < 8; ++u) dots[u] = 0.f;
 #pragma unroll
-        for (int i = 0; i < VEC / 2; ++i) dot = dot2_bf16(xw[i], ww[i], dot);
-        if (late_scale) {  // uniform
-          // a bf16 val widened to fp32 keeps its 16 bits in the upper half
-          const uint32_t v_hi = static_cast<uint32_t>(bcast_i32(static_cast<int>(vbits), j + u));
-          const uint32_t v_lo = v_hi >> 16;
+    for (int h = 0; h < 8; h += FLEXSAE_TOPK_ROWS_PER_TEST) {
+      if (h != 0 && j + h >= n) continue;  // uniform
 #pragma unroll
-          for (int i = 0; i < VEC / 2; ++i) {
-            acc[2 * i] = dot2_bf16(xw[i], v_lo, acc[2 * i]);
-            acc[2 * i + 1] = dot2_bf16(xw[i], v_hi, acc[2 * i + 1]);
+      for (int u = h; u < h + FLEXSAE_TOPK_ROWS_PER_TEST; ++u) {
+        float dot = 0.f;
+        if constexpr (kDot2) {
+          uint32_t xw[VEC / 2];
+          __builtin_memcpy(xw, &rows[u], sizeof(xw));
+#pragma unroll
+          for (int i = 0; i < VEC / 2; ++i) dot = dot2_bf16(xw[i], ww[i], dot);
+          if (late_scale) {  // uniform
+            // a bf16 val widened to fp32 keeps its 16 bits in the upper half
+            const uint32_t v_hi = static_cast<uint32_t>(bcast_i32(static_cast<int>(vbits), j + u));
+            const uint32_t v_lo = v_hi >> 16;
+#pragma unroll
+            for (int i = 0; i < VEC / 2; ++i) {
+              acc[2 * i] = dot2_bf16(xw[i], v_lo, acc[2 * i]);
+              acc[2 * i + 1] = dot2_bf16(xw[i], v_hi, acc[2 * i + 1]);
+            }
+          } else {
+            float x[VEC];
+            unpack_raw<RT, VEC>(rows[u], x);
+            const float vj = bcast_f32(v, j + u);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = fmaf(vj, x[i], acc[i]);
           }
         } else {
           float x[VEC];
           unpack_raw<RT, VEC>(rows[u], x);
           const float vj = bcast_f32(v, j + u);
 #pragma unroll
-          for (int i = 0; i < VEC; ++i) acc[i] = fmaf(vj, x[i], acc[i]);
+          for (int i = 0; i < VEC; ++i) {
+            acc[i] = fmaf(vj, x[i], acc[i]);
+            dot = fmaf(x[i], w[i], dot);
+          }
         }
-      } else {
-        float x[VEC];
-        unpack_raw<RT, VEC>(rows[u], x);
-        const float vj = bcast_f32(v, j + u);
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          acc[i] = fmaf(vj, x[i], acc[i]);
-          dot = fmaf(x[i], w[i], dot);
-        }
+        dots[u] = dot;
       }
-      dots[u] = dot;
     }
     const float tot = wave_sum8_transposed(dots);  // lane L: total of slot j + (L & 7)
     if ((lane >> 3) == (j >> 3)) my_dot = tot;
