@@ -6,9 +6,16 @@ Op graph (names under the ``flexsae_amd::`` namespace):
     hier_bwd(grad_out, indices, weight, vals, resid) -> (dW, dvals, dbias)
     topk_fwd(indices, weight, vals, bias, target) -> (loss, resid)
     topk_bwd(grad_out, indices, weight, vals, resid) -> (dW, dvals, dbias)
+    hier_train_sliced(indices, weight, vals, bias, target) -> (loss, dvals, dbias, dW)   [unit gradient]
+    scale_(x, grad_out), scale_by(x, grad_out) -> x * grad_out
+    hier_train(indices, weight, vals, bias, target) -> (loss, dvals, dbias, stage)       [unit gradient]
+    hier_finish(grad_out, indices, weight, vals, stage) -> dW
 
-``resid[B,D]`` (fp32) is the reconstruction error of the full row, the only state kept between
-forward and backward.  The ops take the place of the reference's two ``autograd.Function``
+``resid[B,D]`` (fp32) is the reconstruction error of the full row, the only state the first four
+keep between forward and backward.  The hierarchical loss, when gradients are needed, goes
+through ``hier_train_sliced`` instead (forward and reverse walk sharing one gather; the backward
+only scales), or through ``hier_train`` / ``hier_finish`` when a stage budget lets all per-pair
+contributions wait for the backward.  The ops take the place of the reference's two ``autograd.Function``
 classes (reference torch-ext/flex_sae/hierarchical_kernels.py:273-299 and
 torch-ext/flex_sae/topk_kernels.py:188-223) and keep their contract: gradients for ``weight``,
 ``vals`` and ``bias`` only (plus ``target`` for TopK, whose loss tail is differentiable there),
