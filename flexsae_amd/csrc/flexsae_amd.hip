@@ -443,6 +443,34 @@ size_t hier_bwd_bytes(const HierBwdPlan &p, int64_t slice_w) {
          round_up(p.n_pairs * static_cast<size_t>(slice_w) * p.p_size, kAlign);
 }
 
+// Segment reduction of one slice plus the finalize step of its hot latents.  fp32 contributions
+// are read 16 bytes per lane (256-column tiles), or, when `narrow`, 8 bytes per lane (128-column
+// tiles, twice the wavefronts): faster once a latent has about four rows or more, slower for
+// shorter groups.
+template <typename PT, typename GT, int VEC>
+void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc, const uint32_t *chunk_begin,
+                       const void *P, float *partial, void *dW, const float *dw_scale, int64_t F, int tps,
+                       int col0, int sw, int D, hipStream_t st) {
+  constexpr bool kCanNarrow = sizeof(typename Traits<PT>::store_t) == 4 && VEC == 4;
+  if (kCanNarrow && narrow) {
+    constexpr int RV = kCanNarrow ? 2 : VEC;
+    const int rtps = tps * (VEC / RV);
+    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(F * rtps, kWavesPerBlock));
+    hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, RV, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks),
+                       dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale,
+                       F, kLongBlocks, rtps, col0, sw, D);
+    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, RV, 8>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
+                       sc.long_list, chunk_begin, partial, dW, dw_scale, rtps, col0, sw, D);
+    return;
+  }
+  const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(F * tps, kWavesPerBlock));
+  hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks),
+                     dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, F,
+                     kLongBlocks, tps, col0, sw, D);
+  hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
+                     sc.long_list, chunk_begin, partial, dW, dw_scale, tps, col0, sw, D);
+}
+
 template <typename WT, typename PT, typename GT, int VEC>
 void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t slice_w,
                         const int64_t *indices, const void *weight, const void *vals,
@@ -465,6 +493,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const int d_pad = static_cast<int>(pl.d_pad);
   const int K = static_cast<int>(s->K), D = static_cast<int>(s->D);
   const int sw = static_cast<int>(slice_w);
+  const bool narrow_reduce = s->B * s->K >= 4 * s->F;
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
@@ -480,13 +509,8 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                          s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F,
                          D);
     if (!do_reduce) continue;
-    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(s->F * tps, kWavesPerBlock));
-    hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks), dim3(kBlock),
-                       0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, s->F,
-                       kLongBlocks, tps, static_cast<int>(col0), sw, D);
-    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st,
-                       sc.long_count, sc.long_list, chunk_begin, partial, dW, dw_scale, tps,
-                       static_cast<int>(col0), sw, D);
+    launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
+                                   static_cast<int>(col0), sw, D, st);
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
