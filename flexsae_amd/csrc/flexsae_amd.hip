@@ -331,6 +331,12 @@ void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
                        slot);
 }
 
+// Columns per tile of the training-step kernel: one register per gathered row piece, so 16-bit
+// weights take two columns per lane (128-column tiles) and fp32 weights one once K exceeds 64.
+inline int64_t train_tile_cols(const flexsae_shape *s) {
+  return (s->weight_dtype == FLEXSAE_F32 && s->K > 64) ? 64 : 128;
+}
+
 // ---- two-phase hierarchical backward: workspace plan -----------------------------------
 
 struct HierBwdPlan {
@@ -342,7 +348,7 @@ struct HierBwdPlan {
   size_t n_rows;           // B
   size_t n_partial_rows;   // upper bound on the number of 64-pair chunks of long latents
   size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_sfinal, off_colsum, off_loss, off_dvpart, off_partial;  // per-slice buffers follow
-  size_t n_loss_partials;  // training-step kernel: one per (128-column tile, row)
+  size_t n_loss_partials;  // training-step kernel: one per (tile of 64 or 128 columns, row)
   size_t fixed_bytes;      // everything that does not depend on the slice width
 };
 
@@ -371,12 +377,13 @@ HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
   p.off_colsum = off;  // partial column sums, [ceil(B/64), D] fp32
   off += round_up(static_cast<size_t>(ceil_div(s->B, kColsumRows)) * static_cast<size_t>(s->D) * 4, kAlign);
   p.off_loss = off;
-  p.n_loss_partials = p.n_rows * static_cast<size_t>(p.d_pad / 128 + 1);
+  p.n_loss_partials = p.n_rows * static_cast<size_t>(p.d_pad / 64 + 1);
   off += round_up(p.n_loss_partials * 4, kAlign);
   // per-tile shares of dvals, [number of tiles, B*K] fp32, added up in tile order afterwards
-  // (tiles are 128 columns in the training-step kernel, 64*vec in the sweep kernel)
+  // (tiles are 64 or 128 columns in the training-step kernel, 64*vec in the sweep kernel)
   p.off_dvpart = off;
-  off += round_up(static_cast<size_t>(p.d_pad / (p.tile < 128 ? p.tile : 128)) * p.n_pairs * 4, kAlign);
+  const int64_t tt = train_tile_cols(s);
+  off += round_up(static_cast<size_t>(p.d_pad / (p.tile < tt ? p.tile : tt)) * p.n_pairs * 4, kAlign);
   p.off_partial = off;
   p.fixed_bytes = off;
   return p;
@@ -389,23 +396,21 @@ struct TrainArgs {
 };
 
 // largest K the training-step kernel holds in registers, per weight dtype
-inline int train_kmax(int weight_dtype) { return weight_dtype == FLEXSAE_F32 ? 64 : 128; }
-inline bool train_supported(const flexsae_shape *s) {
-  return s->D % 4 == 0 && s->K <= train_kmax(s->weight_dtype);
-}
+inline bool train_supported(const flexsae_shape *s) { return s->D % 4 == 0 && s->K <= 128; }
 
-template <typename WT, typename PT, int KMAX>
+template <typename WT, typename PT, int KMAX, int VEC = 2>
 void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
                          const void *weight, const void *vals, float coef, const uint32_t *slot, void *P,
                          float *dvals, float *s_final, int d_pad, float *loss_partial, int *status_flag,
                          int64_t cols, int col0, int slice_w, hipStream_t st) {
-  const int64_t n_items = s->B * (cols / 128);
+  const int64_t n_items = s->B * (cols / (kWave * VEC));
   // K == KMAX (the usual powers of two) runs the variant without per-step bound tests
   const bool stream = slice_w >= d_pad;  // all of P in one launch: streaming stores
   const auto kernel = s->K == KMAX
-                          ? (stream ? hier_train_kernel<WT, PT, KMAX, true, true> : hier_train_kernel<WT, PT, KMAX, true, false>)
-                          : (stream ? hier_train_kernel<WT, PT, KMAX, false, true>
-                                    : hier_train_kernel<WT, PT, KMAX, false, false>);
+                          ? (stream ? hier_train_kernel<WT, PT, KMAX, true, true, VEC>
+                                    : hier_train_kernel<WT, PT, KMAX, true, false, VEC>)
+                          : (stream ? hier_train_kernel<WT, PT, KMAX, false, true, VEC>
+                                    : hier_train_kernel<WT, PT, KMAX, false, false, VEC>);
   hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
                      indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
                      coef, slot, P, dvals, s_final, d_pad, loss_partial, status_flag, n_items, s->B, col0,
@@ -427,8 +432,11 @@ void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const in
     FLEXSAE_TRAIN(32);
   } else if (s->K <= 64) {
     FLEXSAE_TRAIN(64);
-  } else {
-    if constexpr (sizeof(typename Traits<WT>::store_t) == 2) FLEXSAE_TRAIN(128);
+  } else if constexpr (sizeof(typename Traits<WT>::store_t) == 2) {
+    FLEXSAE_TRAIN(128);
+  } else {  // fp32 rows of 65..128 steps: one column per lane
+    launch_train_kernel<WT, PT, 128, 1>(s, ta, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,
+                                        loss_partial, status_flag, cols, col0, slice_w, st);
   }
 #undef FLEXSAE_TRAIN
 }
@@ -516,7 +524,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
   // dvals = its per-tile shares added in tile order
   hipLaunchKernelGGL(hier_dvals_finalize_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, dv_part,
-                     static_cast<int>(pl.d_pad / (train ? 128 : pl.tile)), s->B * s->K, dvals);
+                     static_cast<int>(pl.d_pad / (train ? train_tile_cols(s) : pl.tile)), s->B * s->K, dvals);
   // dbias = column sums of s_final over the rows, in a fixed order
   hipLaunchKernelGGL(colsum_partial_kernel,
                      dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
@@ -925,7 +933,7 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   rc = launch_status();
   if (rc != FLEXSAE_OK) return rc;
   hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(1024), 0, st,
-                     reinterpret_cast<const float *>(ws + pl.off_loss), s->B * (pl.d_pad / 128), 1.0 / count,
+                     reinterpret_cast<const float *>(ws + pl.off_loss), s->B * (pl.d_pad / train_tile_cols(s)), 1.0 / count,
                      loss);
   return launch_status();
 }

@@ -5,11 +5,11 @@
 
 namespace flexsae {
 
-// A gathered piece of a weight row (two consecutive columns) kept in raw form.
-template <typename WT>
-struct RowPiece2;
+// A gathered piece of a weight row (VEC consecutive columns of one lane) kept in raw form.
+template <typename WT, int VEC>
+struct RowPiece;
 template <>
-struct RowPiece2<float> {
+struct RowPiece<float, 2> {
   using raw_t = vec_t<float, 2>;
   static __device__ __forceinline__ void unpack(const raw_t &r, float (&w)[2]) {
     w[0] = r[0];
@@ -19,7 +19,13 @@ struct RowPiece2<float> {
   static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
 };
 template <>
-struct RowPiece2<bf16_t> {
+struct RowPiece<float, 1> {
+  using raw_t = float;
+  static __device__ __forceinline__ void unpack(const raw_t &r, float (&w)[1]) { w[0] = r; }
+  static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
+};
+template <>
+struct RowPiece<bf16_t, 2> {
   using raw_t = uint32_t;
   static __device__ __forceinline__ void unpack(const raw_t &r, float (&w)[2]) {
     w[0] = __uint_as_float(r << 16);
@@ -28,7 +34,7 @@ struct RowPiece2<bf16_t> {
   static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
 };
 template <>
-struct RowPiece2<f16_t> {
+struct RowPiece<f16_t, 2> {
   using raw_t = uint32_t;
   static __device__ __forceinline__ void unpack(const raw_t &r, float (&w)[2]) {
     w[0] = f16_bits_to_f32(static_cast<uint16_t>(r & 0xffffu));
@@ -37,8 +43,10 @@ struct RowPiece2<f16_t> {
   static __device__ __forceinline__ void launder(raw_t &r) { asm volatile("" : "+v"(r)); }
 };
 
-// One wavefront per (tile of the slice, row b), tile-major; a tile is 128 columns and lane l owns
-// columns 2l, 2l+1.  The wavefront issues the gathers of all K row pieces at once (the memory
+// One wavefront per (tile of the slice, row b), tile-major; a tile is 64*VEC columns and lane l owns
+// columns VEC*l .. VEC*l+VEC-1 (VEC = 2: 128-column tiles, 256 bytes of a 16-bit row per gather;
+// VEC = 1, for fp32 weights with more than 64 steps: 64-column tiles, again 256 bytes and one
+// register per row).  The wavefront issues the gathers of all K row pieces at once (the memory
 // pipeline keeps up to 63 of them in flight per wavefront, so a few wavefronts per SIMD cover the
 // latency), keeps the pieces in registers -- one register per row for 16-bit weights -- and walks
 // them twice:
@@ -56,7 +64,7 @@ struct RowPiece2<f16_t> {
 // when all of P is written before any of it is read back (it is far larger than the caches);
 // when P is one slice that the reduction reads right after this launch, plain stores leave part
 // of it in the memory-side cache and the pair of launches is faster.
-template <typename WT, typename PT, int KMAX, bool FULL, bool STREAM>
+template <typename WT, typename PT, int KMAX, bool FULL, bool STREAM, int VEC>
 __global__ __launch_bounds__(256) void hier_train_kernel(
     const int64_t *__restrict__ indices, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
@@ -64,10 +72,9 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     const uint32_t *__restrict__ slot, void *__restrict__ P, float *__restrict__ dv_part,
     float *__restrict__ s_final, int s_final_ld, float *__restrict__ loss_partial,
     int *status_flag, int64_t n_items, int64_t B, int col0, int slice_w, int K, int64_t F, int D) {
-  using Piece = RowPiece2<WT>;
+  using Piece = RowPiece<WT, VEC>;
   using raw_t = typename Piece::raw_t;
   using S_t = typename Traits<WT>::store_t;
-  constexpr int VEC = 2;
   constexpr int KC = (KMAX + kWave - 1) / kWave;  // 64-step chunks held per lane
   static_assert(KMAX % 8 == 0, "KMAX must be a multiple of 8");
   const int lane = lane_id();
@@ -150,7 +157,9 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
       }
     }
   }
-  float lsum = active ? (acc[0] + acc[1]) : 0.f;
+  float lsum = 0.f;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) lsum += active ? acc[i] : 0.f;
   lsum = wave_sum_lane63(lsum);
   // one partial per (global tile, row); the finalize kernel adds them in a fixed order
   if (lane == kWave - 1) loss_partial[(static_cast<int64_t>(col0 / (kWave * VEC)) + t) * B + b] = lsum;
@@ -189,11 +198,12 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
           }
           vec_t<uint32_t, VEC * sizeof(typename Traits<PT>::store_t) / 4> packed;
           if constexpr (Traits<PT>::dtype == FLEXSAE_BF16) {
-            packed[0] = f32x2_to_bf16x2_bits(contrib[0], contrib[1]);
+            static_assert(VEC == 2, "bf16 contributions are stored as pairs");
+            packed[0] = f32x2_to_bf16x2_bits(contrib[0], contrib[VEC - 1]);
           } else {
             static_assert(Traits<PT>::dtype == FLEXSAE_F32, "contributions are staged as bf16 or fp32");
-            packed[0] = __float_as_uint(contrib[0]);
-            packed[1] = __float_as_uint(contrib[1]);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) packed[i] = __float_as_uint(contrib[i]);
           }
           descriptor_store<sizeof(packed), STREAM>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
           dots[u] = dot;  // zero where the lane is beyond column D: its w is zero

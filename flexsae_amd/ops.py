@@ -383,7 +383,7 @@ def set_fused_training(enabled: bool) -> None:
 
 def _train_supported(weight: Tensor, K: int) -> bool:
     D = weight.shape[1]
-    return D % 4 == 0 and K <= (64 if weight.dtype == torch.float32 else 128)
+    return D % 4 == 0 and K <= 128
 
 
 def _stage_fits(indices: Tensor, weight: Tensor) -> bool:
