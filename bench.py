@@ -272,7 +272,7 @@ def main():
                                         p(dvals), p(dbias), p(bws), bws_bytes, flags, None, st()),
                    "flexsae_hier_bwd")
 
-    PRE, REUSE, SWEEP, REDUCE, NO_DW = 1, 2, 4, 8, 32
+    PRE, REUSE, SWEEP, REDUCE, NO_DW, NO_EPILOGUE = 1, 2, 4, 8, 32, 64
     fwd_k_ms = time_kernel_events(torch, lambda: None, fwd_launch, args.steps, args.warmup)
     step_entry_ms = None
     if fused:
@@ -283,9 +283,9 @@ def main():
                                                 st()), "flexsae_hier_fwd_bwd")
 
         step_entry_ms = time_kernel_events(torch, lambda: None, train_launch, args.steps, args.warmup)
-        # the training-step kernel(s) alone: deferred reduction when staged, no dW when sliced
+        # the training-step kernel(s) alone: no pair list (kept), no reductions, no epilogue kernels
         sweep_ms = time_kernel_events(torch, lambda: None,
-                                      lambda: train_launch(PRE | REUSE | (SWEEP if staged else NO_DW)), args.steps, 1)
+                                      lambda: train_launch(PRE | REUSE | NO_DW | NO_EPILOGUE), args.steps, 1)
         reduce_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(PRE | REUSE | REDUCE), args.steps, 1)
         bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
         sweep_name = "hier_train_kernel"

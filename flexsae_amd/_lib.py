@@ -30,6 +30,7 @@ BWD_SWEEP_ONLY = 4
 BWD_REDUCE_ONLY = 8
 BWD_SCALE_BY_GRAD_OUT = 16
 BWD_NO_DW = 32
+BWD_SKIP_EPILOGUE = 64
 
 
 class Shape(ctypes.Structure):

@@ -522,6 +522,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
+  if (flags & FLEXSAE_BWD_SKIP_EPILOGUE) return;
   // dvals = its per-tile shares added in tile order
   hipLaunchKernelGGL(hier_dvals_finalize_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, dv_part,
                      static_cast<int>(pl.d_pad / (train ? train_tile_cols(s) : pl.tile)), s->B * s->K, dvals);
@@ -928,10 +929,11 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   // without dW the reductions are left out like in the deferred case (dW_dtype only selects a template then)
   launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, nullptr, coef, dW,
                           no_dw ? s->weight_dtype : dW_dtype, dvals, dbias, ws,
-                          (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY)) | (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0),
+                          (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE)) |
+                              (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0),
                           status_flag, st, &ta);
   rc = launch_status();
-  if (rc != FLEXSAE_OK) return rc;
+  if (rc != FLEXSAE_OK || (flags & FLEXSAE_BWD_SKIP_EPILOGUE)) return rc;
   hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(1024), 0, st,
                      reinterpret_cast<const float *>(ws + pl.off_loss), s->B * (pl.d_pad / train_tile_cols(s)), 1.0 / count,
                      loss);

@@ -65,9 +65,13 @@ enum {
                                      /* are read (the rest may be NULL): the deferred reduction */
   FLEXSAE_BWD_SCALE_BY_GRAD_OUT = 16,/* deferred reduction only: the contributions were made    */
                                      /* for a unit upstream gradient; multiply dW by grad_out[0]*/
-  FLEXSAE_BWD_NO_DW = 32             /* flexsae_hier_fwd_bwd only: dW is not wanted (may be     */
+  FLEXSAE_BWD_NO_DW = 32,            /* flexsae_hier_fwd_bwd only: dW is not wanted (may be     */
                                      /* NULL); the segment reductions are left out, whatever    */
                                      /* the width of the workspace, and nothing is deferred     */
+  FLEXSAE_BWD_SKIP_EPILOGUE = 64     /* measurement aid for flexsae_hier_fwd_bwd: leave out the */
+                                     /* kernels that finish loss, dvals and dbias (those        */
+                                     /* outputs are then not written), so that a call with      */
+                                     /* NO_DW or SWEEP_ONLY runs the training-step kernel alone */
 };
 
 /* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^29; B*K < 2^32. */

@@ -156,6 +156,10 @@ def test_training_step_without_dw():
         torch.cuda.synchronize()
         assert rc2 == 0 and torch.equal(loss, loss2) and torch.equal(dv, dv2) and torch.equal(db, db2)
         assert torch.isnan(dW2.float()).all()
+    # measurement aid: without the epilogue kernels nothing but the contributions is written
+    rc3, loss3, dW3, dv3, db3 = abi.hier_train(idx, W, v, b, t, dw_dtype=torch.bfloat16, flags=32 | 64)
+    torch.cuda.synchronize()
+    assert rc3 == 0 and torch.isnan(loss3).all() and torch.isnan(dv3).all() and torch.isnan(dW3.float()).all()
 
 
 @pytest.mark.parametrize("stage", [STAGE_ALL, None], ids=["staged", "sliced"])
