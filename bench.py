@@ -256,20 +256,28 @@ def main():
     staged = fused and flex.ops._stage_fits(idx, W)
     hier_mode = "staged" if staged else "sliced" if fused else "unfused"
     slice_cols = D if staged else max(1, scratch // (B * K * p_size))
-    bws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
-    bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
     tile = 64 * (4 if D % 4 == 0 else 2 if D % 2 == 0 else 1)
     d_pad = -(-D // tile) * tile
-    slice_w = min(d_pad, max(tile, -(-slice_cols // tile) * tile))
+    if fused:
+        # slices are whole training tiles when the reduction can work on 256-byte pieces
+        bws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+        train_tile = 64 if (dtype == torch.float32 and K > 64) else 128
+        granule = train_tile if D % (16 // p_size) == 0 else tile
+    else:
+        bws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+        granule = tile
+    bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
+    slice_w = min(d_pad, max(granule, -(-slice_cols // granule) * granule))
     n_slices = -(-D // slice_w)
 
     def fwd_launch():
         _lib.check(lib.flexsae_hier_fwd(ctypes.byref(sh), p(idx), p(W), p(v), p(b), p(t), p(loss), p(resid), p(ws),
                                         ws_bytes, None, st()), "flexsae_hier_fwd")
 
-    def bwd_launch(flags=0):
+    def bwd_launch(flags=0, workspace=None):
+        w = bws if workspace is None else workspace
         _lib.check(lib.flexsae_hier_bwd(ctypes.byref(sh), p(idx), p(W), p(v), p(resid), p(g1), p(dW), DT[dtype],
-                                        p(dvals), p(dbias), p(bws), bws_bytes, flags, None, st()),
+                                        p(dvals), p(dbias), p(w), w.numel(), flags, None, st()),
                    "flexsae_hier_bwd")
 
     PRE, REUSE, SWEEP, REDUCE, NO_DW, NO_EPILOGUE = 1, 2, 4, 8, 32, 64
@@ -286,8 +294,13 @@ def main():
         # the training-step kernel(s) alone: no pair list (kept), no reductions, no epilogue kernels
         sweep_ms = time_kernel_events(torch, lambda: None,
                                       lambda: train_launch(PRE | REUSE | NO_DW | NO_EPILOGUE), args.steps, 1)
-        reduce_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(PRE | REUSE | REDUCE), args.steps, 1)
-        bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
+        reduce_ms = time_kernel_events(torch, lambda: None, lambda: train_launch(PRE | REUSE | REDUCE | NO_EPILOGUE),
+                                       args.steps, 1)
+        # the separate backward entry point (whole 256-column tiles per slice) in a workspace of its own
+        ubws = torch.empty(lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols), dtype=torch.uint8,
+                           device=dev)
+        bwd_k_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(0, ubws), args.steps, args.warmup)
+        del ubws
         sweep_name = "hier_train_kernel"
     elif scratch > 0:
         bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)

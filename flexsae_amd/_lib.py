@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libflexsae_amd.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # flexsae_status
 OK = 0
@@ -63,6 +63,7 @@ SIGNATURES = {
     "flexsae_hier_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_hier_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p, _p]),
     "flexsae_hier_fwd_bwd_supported": (_int, [_shape_p]),
+    "flexsae_hier_fwd_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_hier_fwd_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p, _p]),
     "flexsae_scale": (_int, [_p, _p, _int, _i64, _p, _p]),
     "flexsae_hier_bwd_atomic": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p]),

@@ -389,6 +389,18 @@ HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
   return p;
 }
 
+// Slice granule (columns) of the training step.  The training-step kernel works on tiles of
+// train_tile_cols(); when dW rows can be written 16 bytes per lane, the reduction works on
+// 256-byte pieces of P (seg_reduce_piece_kernel) and a slice may be any number of training tiles
+// wide; otherwise slices are whole reduction tiles (64 * vec columns).
+inline int64_t piece_cols(const HierBwdPlan &p) { return kPieceBytes / static_cast<int64_t>(p.p_size); }
+
+inline bool piece_reduce_ok(const flexsae_shape *s, const HierBwdPlan &p, const void *dW, int dW_dtype) {
+  const int64_t ev = 16 / static_cast<int64_t>(p.p_size);  // columns per lane of the piece reduction
+  return s->D % ev == 0 && train_tile_cols(s) % piece_cols(p) == 0 &&
+         (dW == nullptr || aligned(dW, static_cast<size_t>(ev) * dtype_size(dW_dtype)));
+}
+
 // Forward-only inputs of the training-step variant of the slice loop (null = plain backward).
 struct TrainArgs {
   const void *bias;
@@ -458,7 +470,18 @@ size_t hier_bwd_bytes(const HierBwdPlan &p, int64_t slice_w) {
 template <typename PT, typename GT, int VEC>
 void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc, const uint32_t *chunk_begin,
                        const void *P, float *partial, void *dW, const float *dw_scale, int64_t F, int tps,
-                       int col0, int sw, int D, hipStream_t st) {
+                       int col0, int sw, int D, hipStream_t st, int piece_cols = 0, int64_t cols = 0) {
+  if (piece_cols > 0) {  // 256-byte pieces, sixteen lanes each
+    const int pps = static_cast<int>(cols / piece_cols);
+    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(F * pps, kBlock / kPieceLanes));
+    hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks),
+                       dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale,
+                       F, kLongBlocks, pps, col0, sw, D);
+    // the chunk partials of hot latents are combined per 64-column tile
+    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, 1, 8>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
+                       sc.long_list, chunk_begin, partial, dW, dw_scale, static_cast<int>(cols / kWave), col0, sw, D);
+    return;
+  }
   constexpr bool kCanNarrow = sizeof(typename Traits<PT>::store_t) == 4 && VEC == 4;
   if (kCanNarrow && narrow) {
     constexpr int RV = kCanNarrow ? 2 : VEC;
@@ -484,7 +507,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                         const int64_t *indices, const void *weight, const void *vals,
                         const float *resid, const float *grad_out, float coef, void *dW,
                         float *dvals, float *dbias, uint8_t *ws, int flags, int *status_flag,
-                        hipStream_t st, const TrainArgs *train = nullptr) {
+                        hipStream_t st, const TrainArgs *train = nullptr, int piece = 0) {
   const bool do_sweep = !(flags & FLEXSAE_BWD_REDUCE_ONLY);
   const bool do_reduce = !(flags & FLEXSAE_BWD_SWEEP_ONLY);
   const float *dw_scale = (flags & FLEXSAE_BWD_SCALE_BY_GRAD_OUT) ? grad_out : nullptr;
@@ -492,8 +515,6 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const uint32_t *slot = reinterpret_cast<const uint32_t *>(ws + pl.off_slot);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
   uint32_t *chunk_begin = reinterpret_cast<uint32_t *>(ws + pl.off_chunk);
-  float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
-  void *P = ws + pl.off_partial + hier_partial_bytes(pl, slice_w);
   float *s_final = reinterpret_cast<float *>(ws + pl.off_sfinal);
   float *dv_part = reinterpret_cast<float *>(ws + pl.off_dvpart);
   float *colsum_part = reinterpret_cast<float *>(ws + pl.off_colsum);
@@ -502,6 +523,8 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const int K = static_cast<int>(s->K), D = static_cast<int>(s->D);
   const int sw = static_cast<int>(slice_w);
   const bool narrow_reduce = s->B * s->K >= 4 * s->F;
+  float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
+  void *P = ws + pl.off_partial + hier_partial_bytes(pl, slice_w);
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
@@ -518,7 +541,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                          D);
     if (!do_reduce) continue;
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
-                                   static_cast<int>(col0), sw, D, st);
+                                   static_cast<int>(col0), sw, D, st, piece, cols);
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
@@ -539,19 +562,19 @@ void launch_hier_slices_g(const flexsae_shape *s, const HierBwdPlan &pl, int64_t
                           const int64_t *indices, const void *weight, const void *vals,
                           const float *resid, const float *grad_out, float coef, void *dW,
                           int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int flags,
-                          int *status_flag, hipStream_t st, const TrainArgs *train) {
+                          int *status_flag, hipStream_t st, const TrainArgs *train, int piece) {
   switch (dW_dtype) {
     case FLEXSAE_F32:
       launch_hier_slices<WT, PT, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                             coef, dW, dvals, dbias, ws, flags, status_flag, st, train);
+                                             coef, dW, dvals, dbias, ws, flags, status_flag, st, train, piece);
       break;
     case FLEXSAE_BF16:
       launch_hier_slices<WT, PT, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dvals, dbias, ws, flags, status_flag, st, train);
+                                              coef, dW, dvals, dbias, ws, flags, status_flag, st, train, piece);
       break;
     default:
       launch_hier_slices<WT, PT, f16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                             coef, dW, dvals, dbias, ws, flags, status_flag, st, train);
+                                             coef, dW, dvals, dbias, ws, flags, status_flag, st, train, piece);
   }
 }
 
@@ -560,19 +583,19 @@ void launch_hier_slices_w(const flexsae_shape *s, const HierBwdPlan &pl, int64_t
                           const int64_t *indices, const void *weight, const void *vals,
                           const float *resid, const float *grad_out, float coef, void *dW,
                           int dW_dtype, float *dvals, float *dbias, uint8_t *ws, int flags,
-                          int *status_flag, hipStream_t st, const TrainArgs *train = nullptr) {
+                          int *status_flag, hipStream_t st, const TrainArgs *train = nullptr, int piece = 0) {
   switch (s->weight_dtype) {
     case FLEXSAE_F32:
       launch_hier_slices_g<float, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train);
+                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train, piece);
       break;
     case FLEXSAE_BF16:
       launch_hier_slices_g<bf16_t, bf16_t, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                                coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train);
+                                                coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train, piece);
       break;
     default:
       launch_hier_slices_g<f16_t, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
-                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train);
+                                              coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train, piece);
   }
 }
 
@@ -788,6 +811,15 @@ size_t flexsae_hier_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_co
   return hier_bwd_bytes(pl, sw);
 }
 
+size_t flexsae_hier_fwd_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_cols) {
+  if (check_shape(s) != FLEXSAE_OK || !train_supported(s)) return 0;
+  const HierBwdPlan pl = plan_hier_bwd(s);
+  const int64_t granule = piece_reduce_ok(s, pl, nullptr, s->weight_dtype) ? train_tile_cols(s) : pl.tile;
+  int64_t sw = slice_cols <= 0 ? granule : ceil_div(slice_cols, granule) * granule;
+  if (sw > pl.d_pad) sw = pl.d_pad;
+  return hier_bwd_bytes(pl, sw);
+}
+
 int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void *weight,
                      const void *vals, const float *resid, const float *grad_out, void *dW,
                      int dW_dtype, float *dvals, float *dbias, void *workspace,
@@ -906,11 +938,15 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
       (!defer_reduce && !no_dw && !aligned(dW, 4 * dtype_size(dW_dtype))) || !aligned(dvals, 16) ||
       !aligned(dbias, 16))
     return FLEXSAE_ERR_ALIGNMENT;
-  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, pl.tile))
+  // slices are whole training tiles when the reduction can work on 256-byte pieces, else whole
+  // reduction tiles
+  const bool piece = piece_reduce_ok(s, pl, (defer_reduce || no_dw) ? nullptr : dW, dW_dtype);
+  const int64_t granule = piece ? train_tile_cols(s) : pl.tile;
+  if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, granule))
     return FLEXSAE_ERR_WORKSPACE;
-  int64_t slice_w = pl.tile;
-  while (slice_w + pl.tile <= pl.d_pad && hier_bwd_bytes(pl, slice_w + pl.tile) <= workspace_bytes)
-    slice_w += pl.tile;
+  int64_t slice_w = granule;
+  while (slice_w + granule <= pl.d_pad && hier_bwd_bytes(pl, slice_w + granule) <= workspace_bytes)
+    slice_w += granule;
   if (defer_reduce && slice_w < pl.d_pad) return FLEXSAE_ERR_WORKSPACE;  // contributions must all fit
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint8_t *ws = static_cast<uint8_t *>(workspace);
@@ -931,7 +967,7 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
                           no_dw ? s->weight_dtype : dW_dtype, dvals, dbias, ws,
                           (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE)) |
                               (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0),
-                          status_flag, st, &ta);
+                          status_flag, st, &ta, piece ? static_cast<int>(piece_cols(pl)) : 0);
   rc = launch_status();
   if (rc != FLEXSAE_OK || (flags & FLEXSAE_BWD_SKIP_EPILOGUE)) return rc;
   hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(1024), 0, st,

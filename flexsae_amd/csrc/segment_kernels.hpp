@@ -120,6 +120,94 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
   }
 }
 
+// Same reduction with a finer work item: sixteen lanes (a quarter of a wavefront), 16 bytes each,
+// serve one (latent, 256-byte piece of the slice's rows of P) -- 128 columns of bf16 contributions,
+// 64 of fp32 -- so that a slice may be any whole number of such pieces wide.  A narrow slice is what
+// keeps the contributions of one slice in the memory-side cache between the launch that writes them
+// and this one.  The four latents (or pieces) of a wavefront have different row counts: the loop
+// runs to the longest, loads beyond a group's own count are masked off.  Work order: pieces of a
+// latent adjacent, latents ascending, so the launch still reads P front to back.
+constexpr int kPieceLanes = 16;
+constexpr int kPieceBytes = kPieceLanes * 16;
+
+template <typename PT, typename GT, int U>
+__global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
+    const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
+    const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
+    const void *__restrict__ P, float *__restrict__ partial, void *__restrict__ out,
+    const float *__restrict__ scale, int64_t F, unsigned n_long_blocks, int pps, int col0,
+    int slice_w, int D) {
+  using S = typename Traits<PT>::store_t;
+  constexpr int EV = 16 / static_cast<int>(sizeof(S));  // columns per lane
+  constexpr int kGroupsPerBlock = 256 / kPieceLanes;
+  const int sub = static_cast<int>(threadIdx.x) & (kPieceLanes - 1);
+  const int group = static_cast<int>(threadIdx.x) / kPieceLanes;
+  const S *__restrict__ Pp = static_cast<const S *>(P);
+
+  // acc += rows [r0, r0+n) of P at the lane's columns; n differs between the groups of a wavefront
+  auto accumulate = [&](int64_t r0, int n, int pc, float (&acc)[EV]) {
+    const S *row = Pp + r0 * slice_w + pc;
+    for (int j = 0; __any(j < n); j += U) {
+      raw_vec_t<PT, EV> raw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        raw[u] = raw_vec_t<PT, EV>{};
+        if (j + u < n)
+          raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw_vec_t<PT, EV> *>(row + static_cast<int64_t>(j + u) * slice_w));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float x[EV];
+        unpack_raw<PT, EV>(raw[u], x);
+#pragma unroll
+        for (int i = 0; i < EV; ++i) acc[i] += x[i];  // masked-off loads left zeros
+      }
+    }
+  };
+
+  if (blockIdx.x >= n_long_blocks) {
+    const int64_t item = static_cast<int64_t>(blockIdx.x - n_long_blocks) * kGroupsPerBlock + group;
+    const int64_t f = item / pps;
+    const int t = static_cast<int>(item - f * pps);
+    uint32_t s0 = 0, n = 0;
+    if (f < F) {
+      s0 = begin[f];
+      n = begin[f + 1] - s0;
+    }
+    const bool mine = f < F && n <= static_cast<uint32_t>(kSegChunk);  // longer ones: chunked below
+    const int pc = t * (kPieceLanes * EV) + sub * EV;
+    const int d0 = col0 + pc;
+    float acc[EV];
+#pragma unroll
+    for (int i = 0; i < EV; ++i) acc[i] = 0.f;
+    accumulate(s0, mine ? static_cast<int>(n) : 0, pc, acc);
+    if (scale) {  // the rows were produced for a unit upstream gradient
+      const float g = scale[0];
+#pragma unroll
+      for (int i = 0; i < EV; ++i) acc[i] *= g;
+    }
+    if (mine && d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
+    return;
+  }
+  const uint32_t n_long = *long_count;
+  if (n_long == 0) return;
+  const int64_t total = static_cast<int64_t>(chunk_begin[n_long]) * pps;
+  const int64_t n_groups = static_cast<int64_t>(n_long_blocks) * kGroupsPerBlock;
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * kGroupsPerBlock + group; __any(w < total); w += n_groups) {
+    const bool valid = w < total;
+    const int64_t ww = valid ? w : 0;
+    const uint32_t chunk = static_cast<uint32_t>(ww / pps);
+    const int t = static_cast<int>(ww - static_cast<int64_t>(chunk) * pps);
+    const LongChunk c = seg_decode_chunk(begin, long_list, chunk_begin, n_long, chunk);
+    const int pc = t * (kPieceLanes * EV) + sub * EV;
+    float acc[EV];
+#pragma unroll
+    for (int i = 0; i < EV; ++i) acc[i] = 0.f;
+    accumulate(c.s0, valid ? static_cast<int>(c.s1 - c.s0) : 0, pc, acc);
+    if (valid) store_vec<float, EV>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
+  }
+}
+
 // Long latents, second launch: out[f, slice] = sum of the latent's chunk partials, in chunk order.
 template <typename GT, int VEC, int U>
 __global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(

@@ -508,7 +508,7 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
         p_size = 2 if weight.dtype == torch.bfloat16 else 4
         slice_cols = max(1, _hier_scratch_bytes // (B * K * p_size))
-        ws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
+        ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         dW = torch.empty_like(weight)

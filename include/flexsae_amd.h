@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define FLEXSAE_ABI_VERSION 1
+#define FLEXSAE_ABI_VERSION 2
 
 typedef enum {
   FLEXSAE_OK = 0,
@@ -165,8 +165,17 @@ int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const v
  * price is that the workspace (B*K*D contributions) must stay alive in between.
  * With FLEXSAE_BWD_NO_DW (a decoder whose weight needs no gradient) the reductions are left out
  * for any workspace width: loss, dvals and dbias as usual, dW untouched (may be NULL).
+ * Slicing: the workspace decides the slice width.  flexsae_hier_fwd_bwd_workspace_bytes gives the
+ * bytes for slices of `slice_cols` columns, rounded up to whole training tiles (128 columns for
+ * 16-bit weights, 64 or 128 for fp32) when D is a multiple of the reduction's 16-byte lane width
+ * (8 columns of bf16 contributions, 4 of fp32) -- the reduction then works on 256-byte pieces --
+ * and to whole 256-column tiles otherwise; slice_cols <= 0 asks for the minimum; 0 is returned for
+ * unsupported shapes.  Narrow slices keep one slice of contributions in the memory-side cache
+ * between the kernel that writes it and the reduction that reads it.  A workspace from
+ * flexsae_hier_bwd_workspace_bytes is accepted as well.
  */
 int flexsae_hier_fwd_bwd_supported(const flexsae_shape *shape);
+size_t flexsae_hier_fwd_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slice_cols);
 int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
                          const void *vals, const void *bias, const void *target, float *loss,
                          void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
