@@ -19,6 +19,7 @@ ERR_UNSUPPORTED = -2
 ERR_WORKSPACE = -3
 ERR_LAUNCH = -4
 ERR_ALIGNMENT = -5
+ERR_SCRATCH_LIMIT = -6
 
 # flexsae_dtype
 F32, BF16, F16 = 0, 1, 2
@@ -59,6 +60,7 @@ SIGNATURES = {
     "flexsae_status_string": (ctypes.c_char_p, [_int]),
     "flexsae_fwd_workspace_bytes": (_sz, [_shape_p]),
     "flexsae_hier_fwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _p, _p]),
+    "flexsae_hier_fwd_static": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "flexsae_topk_fwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _p, _p]),
     "flexsae_hier_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_hier_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p, _p]),

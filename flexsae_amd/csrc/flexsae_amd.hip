@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "fwd_kernels.hpp"
 #include "csr_kernels.hpp"
@@ -12,6 +14,13 @@
 #include "topk_bwd_kernels.hpp"
 
 using namespace flexsae;
+
+// Device memory of flexsae_hier_fwd_static, the one entry point that takes no workspace: the
+// forward kernels' per-(row, tile) loss partials live here.  Every GPU the library runs on holds
+// its own copy of the array until the process ends.  Host code never uses the array's name as an
+// address: the per-device address comes from hipGetSymbolAddress (static_scratch_for_current_device).
+constexpr size_t kStaticScratchBytes = FLEXSAE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // gathers in flight per wavefront before the first one is consumed
 #ifndef FLEXSAE_SWEEP_U
@@ -55,6 +64,27 @@ int check_shape(const flexsae_shape *s) {
 }
 
 int launch_status() { return hipGetLastError() == hipSuccess ? FLEXSAE_OK : FLEXSAE_ERR_LAUNCH; }
+
+// Address of `scratch` on the current device, looked up once per device and kept.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch_for_current_device(void **out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FLEXSAE_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return FLEXSAE_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return FLEXSAE_OK;
+}
 
 // Largest vector width (elements per lane) the row layout allows: every row start and
 // every lane offset must be aligned to the vector, and wider than 16 bytes gains nothing.
@@ -740,6 +770,8 @@ const char *flexsae_status_string(int status) {
       return "HIP kernel launch failed";
     case FLEXSAE_ERR_ALIGNMENT:
       return "tensor pointer not aligned to its element size";
+    case FLEXSAE_ERR_SCRATCH_LIMIT:
+      return "problem too large for the static scratch of this entry point (use the variant that takes a workspace)";
     default:
       return "unknown status";
   }
@@ -757,6 +789,21 @@ int flexsae_hier_fwd(const flexsae_shape *shape, const int64_t *indices, const v
                      void *stream) {
   return forward<true>(shape, indices, weight, vals, bias, target, loss, resid, workspace,
                        workspace_bytes, status_flag, stream);
+}
+
+int flexsae_hier_fwd_static(const flexsae_shape *shape, const int64_t *indices, const void *weight,
+                            const void *vals, const void *bias, const void *target, float *loss,
+                            float *resid, int *status_flag, void *stream) {
+  const int rc = check_shape(shape);
+  if (rc != FLEXSAE_OK) return rc;
+  if (flexsae_fwd_workspace_bytes(shape) > kStaticScratchBytes) return FLEXSAE_ERR_SCRATCH_LIMIT;
+  void *ptr = nullptr;
+  const int src = static_scratch_for_current_device(&ptr);
+  if (src != FLEXSAE_OK) return src;
+  // every partial the finalize kernel reads is written by the forward kernel of the same call:
+  // nothing in the array has to start at zero
+  return forward<true>(shape, indices, weight, vals, bias, target, loss, resid, ptr, kStaticScratchBytes,
+                       status_flag, stream);
 }
 
 int flexsae_topk_fwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,

@@ -4,7 +4,8 @@
  *
  * Every entry point takes raw device pointers and sizes, launches its kernels on
  * the given HIP stream and returns immediately (no allocation, no
- * synchronisation, no host<->device copy, no global state).  Return value:
+ * synchronisation, no host<->device copy, no global state -- except the static
+ * scratch array of flexsae_hier_fwd_static).  Return value:
  * FLEXSAE_OK or a negative flexsae_status; nothing throws or aborts.
  *
  * Conventions shared by all entry points
@@ -44,7 +45,8 @@ typedef enum {
   FLEXSAE_ERR_UNSUPPORTED = -2,      /* size beyond what the kernels index (see below) */
   FLEXSAE_ERR_WORKSPACE = -3,        /* workspace missing, too small or misaligned     */
   FLEXSAE_ERR_LAUNCH = -4,           /* the HIP runtime refused a launch               */
-  FLEXSAE_ERR_ALIGNMENT = -5         /* a tensor pointer is not aligned to its element */
+  FLEXSAE_ERR_ALIGNMENT = -5,        /* a tensor pointer is not aligned to its element */
+  FLEXSAE_ERR_SCRATCH_LIMIT = -6     /* problem beyond the static scratch of *_static  */
 } flexsae_status;
 
 typedef enum { FLEXSAE_F32 = 0, FLEXSAE_BF16 = 1, FLEXSAE_F16 = 2 } flexsae_dtype;
@@ -98,6 +100,23 @@ int flexsae_hier_fwd(const flexsae_shape *shape, const int64_t *indices, const v
                      const void *vals, const void *bias, const void *target, float *loss,
                      float *resid, void *workspace, size_t workspace_bytes, int *status_flag,
                      void *stream);
+
+/*
+ * HierarchicalTopK forward for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): flexsae_hier_fwd without the workspace argument.
+ * No counterpart in the reference (its launcher allocates with torch, hierarchical_kernels.py:200-201).
+ * The per-(row, tile) loss partials go to a static device array of FLEXSAE_STATIC_SCRATCH_BYTES
+ * that every GPU the library runs on holds until the process ends; the call allocates nothing
+ * (no hipMalloc/hipFree, no allocating library routine).  Limit: B * ceil(D/64) * 4 bytes must fit
+ * the array (FLEXSAE_ERR_SCRATCH_LIMIT beyond; e.g. B=16384, D=8192 needs 8 MiB).  The first call
+ * on a device looks the array's address up (make it before a graph capture starts).  All calls on
+ * one GPU share the array: calls that overlap in time on one GPU (different streams) race; calls
+ * on one stream are safe.  Outputs are bit-identical to flexsae_hier_fwd's.
+ */
+#define FLEXSAE_STATIC_SCRATCH_BYTES (16u << 20)
+int flexsae_hier_fwd_static(const flexsae_shape *shape, const int64_t *indices, const void *weight,
+                            const void *vals, const void *bias, const void *target, float *loss,
+                            float *resid, int *status_flag, void *stream);
 
 /*
  * TopK forward, fully fused (gather, scale, sum over K, + bias, - target, mean square).

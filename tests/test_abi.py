@@ -35,6 +35,7 @@ def test_header_constants_match_binding():
                         ("FLEXSAE_ERR_WORKSPACE", _lib.ERR_WORKSPACE),
                         ("FLEXSAE_ERR_LAUNCH", _lib.ERR_LAUNCH),
                         ("FLEXSAE_ERR_ALIGNMENT", _lib.ERR_ALIGNMENT),
+                        ("FLEXSAE_ERR_SCRATCH_LIMIT", _lib.ERR_SCRATCH_LIMIT),
                         ("FLEXSAE_BF16", _lib.BF16), ("FLEXSAE_F16", _lib.F16),
                         ("FLEXSAE_ABI_VERSION", _lib.ABI_VERSION)):
         m = re.search(rf"{name}\s*=?\s*(-?\d+)", text)
@@ -42,7 +43,7 @@ def test_header_constants_match_binding():
 
 
 def test_status_strings():
-    for code in (0, -1, -2, -3, -4, -5, -99):
+    for code in (0, -1, -2, -3, -4, -5, -6, -99):
         assert isinstance(_lib.status_string(code), str) and _lib.status_string(code)
 
 
@@ -131,3 +132,15 @@ def test_backward_and_csr_reject_bad_arguments():
     assert lib.flexsae_cast_from_f32(NULL, 1, FAKE, 10, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_cast_from_f32(FAKE, 1, FAKE, -1, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_cast_from_f32(FAKE, 1, FAKE, 0, NULL) == _lib.OK
+
+
+def test_static_forward_rejects_bad_arguments_before_touching_the_gpu():
+    lib = _lib.load()
+    fn = lib.flexsae_hier_fwd_static
+    args = [FAKE] * 7
+    assert fn(ctypes.byref(_shape(B=0)), *args, NULL, NULL) == _lib.ERR_INVALID_ARGUMENT
+    assert fn(ctypes.byref(_shape(F=1 << 31)), *args, NULL, NULL) == _lib.ERR_UNSUPPORTED
+    # B * ceil(D/64) * 4 bytes of loss partials beyond the static array
+    assert fn(ctypes.byref(_shape(B=70000, K=1, D=4096)), *args, NULL, NULL) == _lib.ERR_SCRATCH_LIMIT
+    m = re.search(r"FLEXSAE_STATIC_SCRATCH_BYTES\s*\((\d+)u\s*<<\s*(\d+)\)", open(HEADER).read())
+    assert m and (int(m.group(1)) << int(m.group(2))) == 16 << 20
