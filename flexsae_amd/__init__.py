@@ -9,7 +9,7 @@ Public names mirror reference torch-ext/flex_sae/__init__.py:5-18.  The ``triton
 kept so that existing callers need no edit; nothing here uses Triton.
 """
 from .ops import (check_index_flag, hier_stage_bytes, set_fused_training, set_hier_scratch_bytes, set_hier_stage_bytes,
-                  set_index_checking, shared_pair_list, triton_hierarchical_sae_loss,
+                  set_index_checking, set_topk_residual_bf16, shared_pair_list, triton_hierarchical_sae_loss,
                   triton_topk_sae_loss)
 from .reference import hierarchical_sae_loss, topk_sae_loss
 
@@ -37,5 +37,6 @@ __all__ = [
     "set_hier_stage_bytes",
     "hier_stage_bytes",
     "set_fused_training",
+    "set_topk_residual_bf16",
     "shared_pair_list",
 ]

@@ -32,6 +32,7 @@ BWD_REDUCE_ONLY = 8
 BWD_SCALE_BY_GRAD_OUT = 16
 BWD_NO_DW = 32
 BWD_SKIP_EPILOGUE = 64
+TOPK_BWD_FP32_RESIDUAL = 256
 
 
 class Shape(ctypes.Structure):
@@ -73,7 +74,7 @@ SIGNATURES = {
     "flexsae_csr_build": (_int, [_p, _i64, _i64, _i64, _p, _p, _p, _sz, _p, _p]),
     "flexsae_hier_pair_list_layout": (_int, [_shape_p, ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
     "flexsae_hier_import_pair_list": (_int, [_shape_p, _p, _p, _p, _sz, _p]),
-    "flexsae_topk_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p]),
+    "flexsae_topk_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p]),
     "flexsae_topk_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_cast_from_f32": (_int, [_p, _int, _p, _i64, _p]),
 }

@@ -431,6 +431,14 @@ inline bool piece_reduce_ok(const flexsae_shape *s, const HierBwdPlan &p, const 
          (dW == nullptr || aligned(dW, static_cast<size_t>(ev) * dtype_size(dW_dtype)));
 }
 
+// Columns the slice loop works on: D rounded up to whole reduction tiles, or to whole training tiles
+// when the piece reduction lets slices end there.
+inline int64_t hier_cols_used(const flexsae_shape *s, const HierBwdPlan &p, bool train, bool piece) {
+  if (!(train && piece)) return p.d_pad;
+  const int64_t tt = train_tile_cols(s);
+  return ceil_div(s->D, tt) * tt;
+}
+
 // Forward-only inputs of the training-step variant of the slice loop (null = plain backward).
 struct TrainArgs {
   const void *bias;
@@ -555,8 +563,11 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const bool narrow_reduce = s->B * s->K >= 4 * s->F;
   float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
   void *P = ws + pl.off_partial + hier_partial_bytes(pl, slice_w);
+  // columns that are worked on: whole reduction tiles, or, with the piece reduction, whole training
+  // tiles (tiles that lie entirely beyond column D are left out, and so are their shares below)
+  const int64_t d_used = hier_cols_used(s, pl, train != nullptr, piece != 0);
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
-    const int64_t cols = (pl.d_pad - col0) < slice_w ? (pl.d_pad - col0) : slice_w;
+    const int64_t cols = (d_used - col0) < slice_w ? (d_used - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
     const int64_t sweep_items = s->B * tps;
     if (train && do_sweep) {
@@ -578,7 +589,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   if (flags & FLEXSAE_BWD_SKIP_EPILOGUE) return;
   // dvals = its per-tile shares added in tile order
   hipLaunchKernelGGL(hier_dvals_finalize_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, dv_part,
-                     static_cast<int>(pl.d_pad / (train ? train_tile_cols(s) : pl.tile)), s->B * s->K, dvals);
+                     static_cast<int>(d_used / (train ? train_tile_cols(s) : pl.tile)), s->B * s->K, dvals);
   // dbias = column sums of s_final over the rows, in a fixed order
   hipLaunchKernelGGL(colsum_partial_kernel,
                      dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
@@ -639,11 +650,12 @@ struct TopkBwdPlan {
   bool resid16;  // gather a bf16 copy of the residual (bf16 weights): half the cache footprint
 };
 
-TopkBwdPlan plan_topk_bwd(const flexsae_shape *s) {
+TopkBwdPlan plan_topk_bwd(const flexsae_shape *s, int flags = 0) {
   TopkBwdPlan p;
   // The reference hands its backward the residual gradient in the weight dtype
-  // (topk_kernels.py:52,221); for bf16 weights the gathers here read a bf16 copy as well.
-  p.resid16 = FLEXSAE_TOPK_RESID16 && s->weight_dtype == FLEXSAE_BF16;
+  // (topk_kernels.py:52,221); for bf16 weights the gathers here read a bf16 copy as well, unless
+  // the caller asks for the fp32 residual (the workspace layout of that variant is a subset).
+  p.resid16 = FLEXSAE_TOPK_RESID16 && s->weight_dtype == FLEXSAE_BF16 && !(flags & FLEXSAE_TOPK_BWD_FP32_RESIDUAL);
   p.vec = (s->D % 4 == 0) ? 4 : (s->D % 2 == 0) ? 2 : 1;
   // all-bf16: 16 bytes per lane (512-column tiles) halve the per-tile overheads
   if (FLEXSAE_TOPK_VEC8 && p.resid16 && s->D % 8 == 0) p.vec = 8;
@@ -1018,7 +1030,8 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   rc = launch_status();
   if (rc != FLEXSAE_OK || (flags & FLEXSAE_BWD_SKIP_EPILOGUE)) return rc;
   hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(1024), 0, st,
-                     reinterpret_cast<const float *>(ws + pl.off_loss), s->B * (pl.d_pad / train_tile_cols(s)), 1.0 / count,
+                     reinterpret_cast<const float *>(ws + pl.off_loss),
+                     s->B * (hier_cols_used(s, pl, true, piece) / train_tile_cols(s)), 1.0 / count,
                      loss);
   return launch_status();
 }
@@ -1072,7 +1085,7 @@ size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_co
 }
 
 int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32_t *map,
-                     const void *weight, const void *vals, const float *resid,
+                     const int64_t *indices, const void *weight, const void *vals, const float *resid,
                      const float *grad_out, void *dW, int dW_dtype, float *dvals, float *dbias,
                      void *workspace, size_t workspace_bytes, int flags, void *stream) {
   int rc = check_shape(s);
@@ -1082,8 +1095,9 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
     return FLEXSAE_ERR_INVALID_ARGUMENT;
   // the residual rows are gathered through a 32-bit buffer descriptor
   if (static_cast<size_t>(s->B) * static_cast<size_t>(s->D) * 4 > 0xffffffffull) return FLEXSAE_ERR_UNSUPPORTED;
-  const TopkBwdPlan pl = plan_topk_bwd(s);
-  if (!aligned(begin, 4) || !aligned(map, 4) || !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
+  const TopkBwdPlan pl = plan_topk_bwd(s, flags);
+  if (!aligned(begin, 4) || !aligned(map, 4) || (indices && !aligned(indices, 8)) ||
+      !aligned(weight, pl.vec * dtype_size(s->weight_dtype)) ||
       !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(resid, pl.resid16 ? 16 : pl.vec * 4) ||
       !aligned(grad_out, 4) || !aligned(dW, pl.vec * dtype_size(dW_dtype)) || !aligned(dvals, 16) ||
       !aligned(dbias, 4))
@@ -1095,7 +1109,7 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
     slice_w += pl.tile;
   hipStream_t st = static_cast<hipStream_t>(stream);
   uint8_t *ws = static_cast<uint8_t *>(workspace);
-  (void)flags;  // every output element is written exactly once: nothing needs a zero-fill
+  // (every output element is written exactly once: nothing needs a zero-fill, whatever `flags` says)
   // latents with more than 64 pairs and their chunk table
   uint32_t *long_count = reinterpret_cast<uint32_t *>(ws + pl.off_long_count);
   uint32_t *long_list = reinterpret_cast<uint32_t *>(ws + pl.off_long_list);
@@ -1111,8 +1125,8 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
   {
     const int64_t n_resid = pl.resid16 ? s->B * s->D : 0;
     const int64_t work = s->B * s->K > ceil_div(n_resid, 4) ? s->B * s->K : ceil_div(n_resid, 4);
-    hipLaunchKernelGGL(topk_prepare_kernel, dim3(grid_for(work, 256, 1 << 16)), dim3(256), 0, st, map, vals,
-                       s->vals_dtype, s->B * s->K, static_cast<int>(s->K),
+    hipLaunchKernelGGL(topk_prepare_kernel, dim3(grid_for(work, 256, 1 << 16)), dim3(256), 0, st, map, indices,
+                       s->F, vals, s->vals_dtype, s->B * s->K, static_cast<int>(s->K),
                        reinterpret_cast<vec_t<uint32_t, 2> *>(ws + pl.off_slotbv), resid, n_resid,
                        pl.resid16 ? static_cast<void *>(ws + pl.off_resid16) : nullptr);
   }

@@ -27,9 +27,9 @@ namespace flexsae {
 // B x tile slice of the [B,D] matrix, which has to stay in the 4 MB L2 of every XCD.
 template <typename RT, int VEC>
 __device__ __forceinline__ void topk_accumulate_slots(
-    const uint32_t *__restrict__ map, const void *__restrict__ vals, int vals_dtype,
+    const vec_t<uint32_t, 2> *__restrict__ slot_bv,
     const void *__restrict__ resid, float scale, float *__restrict__ dv_tile, const float (&w)[VEC],
-    uint32_t s_begin, uint32_t s_end, int K, int D, int dsafe, float (&acc)[VEC]) {
+    uint32_t s_begin, uint32_t s_end, int D, int dsafe, float (&acc)[VEC]) {
   using S = typename Traits<RT>::store_t;
   const int lane = lane_id();
   // row address = scalar base of the row + the lane's fixed byte offset
@@ -37,13 +37,13 @@ __device__ __forceinline__ void topk_accumulate_slots(
   const size_t row_bytes = static_cast<size_t>(D) * sizeof(S);
   for (uint32_t s = s_begin; s < s_end; s += kWave) {
     const uint32_t slot = s + lane;
-    uint32_t p = 0;
+    int my_b = 0;
     float v = 0.f;
-    if (slot < s_end) {
-      p = map[slot];
-      v = load_scalar(vals, vals_dtype, p) * scale;
+    if (slot < s_end) {  // the pair's (batch row, val) record; the val of an out-of-range index is zero there
+      const vec_t<uint32_t, 2> bv = slot_bv[slot];
+      my_b = static_cast<int>(bv[0]);
+      v = __uint_as_float(bv[1]) * scale;
     }
-    const int my_b = static_cast<int>(p / static_cast<uint32_t>(K));
     const int n = (s_end - s) < static_cast<uint32_t>(kWave) ? static_cast<int>(s_end - s) : kWave;
     float my_dot = 0.f;
     // eight gathers in flight; a group reaching past the end re-reads the last row (a cache hit);
@@ -278,9 +278,8 @@ __global__ __launch_bounds__(256) void topk_bwd_kernel(
       acc[i] = 0.f;
       if (!active) w[i] = 0.f;
     }
-    topk_accumulate_slots<RT, VEC>(map, vals, vals_dtype, resid, scale,
-                                      dv_part + (col0 / (kWave * VEC) + t) * n_pairs, w, c.s0, c.s1, K, D, dsafe,
-                                      acc);
+    topk_accumulate_slots<RT, VEC>(slot_bv, resid, scale, dv_part + (col0 / (kWave * VEC) + t) * n_pairs, w, c.s0,
+                                   c.s1, D, dsafe, acc);
     store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
   }
 }
@@ -300,9 +299,12 @@ __global__ void topk_dvals_finalize_kernel(const uint32_t *__restrict__ map,
 
 // Preparation of a TopK backward, one launch:
 //   slot_bv[s] = (batch row, val as fp32 bits) of the pair in slot s of the latent-major list: what
-//     the backward reads per pair, contiguous per latent instead of scattered over vals;
+//     the backward reads per pair, contiguous per latent instead of scattered over vals; a pair
+//     whose index lies outside [0, F) gets a val of zero, as in the forward (the pair list files it
+//     under latent 0), so that it adds nothing to dW (`indices` may be null: every val is kept);
 //   resid16[i] = bf16(resid[i]) for i < n_resid (n_resid = 0: no copy wanted).
-__global__ void topk_prepare_kernel(const uint32_t *__restrict__ map, const void *__restrict__ vals,
+__global__ void topk_prepare_kernel(const uint32_t *__restrict__ map, const int64_t *__restrict__ indices,
+                                    int64_t F, const void *__restrict__ vals,
                                     int vals_dtype, int64_t n_pairs, int K,
                                     vec_t<uint32_t, 2> *__restrict__ slot_bv, const float *__restrict__ resid,
                                     int64_t n_resid, void *__restrict__ resid16) {
@@ -312,7 +314,9 @@ __global__ void topk_prepare_kernel(const uint32_t *__restrict__ map, const void
     const uint32_t p = map[s];
     vec_t<uint32_t, 2> r;
     r[0] = p / static_cast<uint32_t>(K);
-    r[1] = __float_as_uint(load_scalar(vals, vals_dtype, p));
+    float v = load_scalar(vals, vals_dtype, p);
+    if (indices && static_cast<uint64_t>(indices[p]) >= static_cast<uint64_t>(F)) v = 0.f;
+    r[1] = __float_as_uint(v);
     slot_bv[s] = r;
   }
   const int64_t n4 = n_resid >> 2;

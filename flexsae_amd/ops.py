@@ -110,6 +110,13 @@ def _shape(B, K, F, D, weight: Tensor, vals: Tensor, bias_dtype, target_dtype) -
                       _DTYPES[target_dtype])
 
 
+def _prep(t: Tensor) -> Tensor:
+    """Contiguous and 16-byte aligned, as the vector accesses of the kernels need: a view into a
+    larger buffer that starts at an odd element (``flat[1:1 + D]``) is copied."""
+    t = t.contiguous()
+    return t.clone() if t.data_ptr() % 16 else t
+
+
 def _ptr(t: Tensor) -> ctypes.c_void_p:
     return ctypes.c_void_p(t.data_ptr())
 
@@ -121,7 +128,7 @@ def _stream() -> ctypes.c_void_p:
 def _forward(entry: str, indices, weight, vals, bias, target) -> Tuple[Tensor, Tensor]:
     B, K, F, D = _validate(indices, weight, vals, bias, target)
     lib = _lib.load()
-    indices, weight, vals, bias, target = (t.contiguous() for t in (indices, weight, vals, bias, target))
+    indices, weight, vals, bias, target = (_prep(t) for t in (indices, weight, vals, bias, target))
     dev = weight.device
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
@@ -269,7 +276,7 @@ def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
     B, K = indices.shape
     F, D = weight.shape
     dev = weight.device
-    indices, weight, vals, resid = (t.contiguous() for t in (indices, weight, vals, resid))
+    indices, weight, vals, resid = (_prep(t) for t in (indices, weight, vals, resid))
     with torch.cuda.device(dev):
         g = _grad_scalar(grad_out, dev)
         shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
@@ -307,6 +314,20 @@ def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
     return dW, dvals, dbias
 
 
+# With bf16 weights the TopK backward gathers a bf16 copy of the residual (half the cache footprint;
+# the reference's backward also receives the residual gradient in the weight dtype, reference
+# torch-ext/flex_sae/topk_kernels.py:52).  That rounding shows in `vals.grad` (about 4e-3 normwise
+# instead of 1e-6); switching it off gathers the fp32 residual instead, a little slower.
+_topk_residual_bf16 = os.environ.get("FLEXSAE_TOPK_RESIDUAL_BF16", "1") not in ("", "0")
+
+
+def set_topk_residual_bf16(enabled: bool) -> None:
+    """bf16 weights only: whether the TopK backward reads a bf16 copy of the residual (default,
+    faster) or the fp32 residual itself (``vals.grad`` then carries fp32 rounding only)."""
+    global _topk_residual_bf16
+    _topk_residual_bf16 = bool(enabled)
+
+
 @torch.library.custom_op("flexsae_amd::topk_bwd", mutates_args=())
 def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
              resid: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
@@ -314,7 +335,7 @@ def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
     B, K = indices.shape
     F, D = weight.shape
     dev = weight.device
-    indices, weight, vals, resid = (t.contiguous() for t in (indices, weight, vals, resid))
+    indices, weight, vals, resid = (_prep(t) for t in (indices, weight, vals, resid))
     with torch.cuda.device(dev):
         g = _grad_scalar(grad_out, dev)
         shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
@@ -338,9 +359,10 @@ def topk_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
         slice_cols = max(1, (256 << 20) // max(1, (B * K // 32) * 4))
         bws_bytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
         bws = torch.empty(bws_bytes, dtype=torch.uint8, device=dev)
-        rc = lib.flexsae_topk_bwd(ctypes.byref(shape), _ptr(begin), _ptr(pair_map), _ptr(weight), _ptr(vals),
-                                  _ptr(resid), _ptr(g), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals),
-                                  _ptr(dbias), _ptr(bws), bws_bytes, 0, _stream())
+        rc = lib.flexsae_topk_bwd(ctypes.byref(shape), _ptr(begin), _ptr(pair_map), _ptr(indices), _ptr(weight),
+                                  _ptr(vals), _ptr(resid), _ptr(g), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals),
+                                  _ptr(dbias), _ptr(bws), bws_bytes,
+                                  0 if _topk_residual_bf16 else _lib.TOPK_BWD_FP32_RESIDUAL, _stream())
         _lib.check(rc, "flexsae_topk_bwd")
     return dW, dvals, dbias
 
@@ -409,7 +431,7 @@ def hier_train(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
     ``hier_finish`` produces dW with the upstream gradient folded in."""
     B, K, F, D = _validate(indices, weight, vals, bias, target)
     lib = _lib.load()
-    indices, weight, vals, bias, target = (t.contiguous() for t in (indices, weight, vals, bias, target))
+    indices, weight, vals, bias, target = (_prep(t) for t in (indices, weight, vals, bias, target))
     dev = weight.device
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
@@ -493,16 +515,17 @@ hier_train.register_autograd(_train_backward, setup_context=_train_setup_context
 
 @torch.library.custom_op("flexsae_amd::hier_train_sliced", mutates_args=())
 def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
-                      target: Tensor) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+                      target: Tensor, need_dw: bool = True) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     """Fused forward + reverse walk in column slices, each reduced right away (flat memory).
 
     Used when the contributions of a whole step do not fit the stage budget: the scratch is one
     slice of them (``set_hier_scratch_bytes``), and every slice gathers its weight-row pieces once
     for both walks.  Returns (loss, dvals, dbias, dW), the gradients for a unit upstream gradient;
-    the backward scales them."""
+    the backward scales them.  With ``need_dw`` false (a decoder whose weight takes no gradient)
+    the segment reductions are left out and the returned dW is empty."""
     B, K, F, D = _validate(indices, weight, vals, bias, target)
     lib = _lib.load()
-    indices, weight, vals, bias, target = (t.contiguous() for t in (indices, weight, vals, bias, target))
+    indices, weight, vals, bias, target = (_prep(t) for t in (indices, weight, vals, bias, target))
     dev = weight.device
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
@@ -511,16 +534,17 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
         ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
-        dW = torch.empty_like(weight)
+        dW = torch.empty_like(weight) if need_dw else weight.new_empty((0, D))
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
         flag = _flag_for(dev)
         cached = _pair_lookup(indices, F)
         if cached is not None:
             _pair_import(lib, shape, workspace, cached)
-        flags = _lib.BWD_REUSE_PAIR_LIST if cached is not None else 0
+        flags = (_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0) | (0 if need_dw else _lib.BWD_NO_DW)
         rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
-                                      _ptr(target), _ptr(loss), _ptr(dW), _DTYPES[weight.dtype], _ptr(dvals),
+                                      _ptr(target), _ptr(loss), _ptr(dW) if need_dw else None,
+                                      _DTYPES[weight.dtype], _ptr(dvals),
                                       _ptr(dbias), _ptr(workspace), ws_bytes, flags, _ptr(flag), _stream())
         _lib.check(rc, "flexsae_hier_fwd_bwd")
         if cached is None:
@@ -531,9 +555,10 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
 
 
 @hier_train_sliced.register_fake
-def _(indices, weight, vals, bias, target):
+def _(indices, weight, vals, bias, target, need_dw=True):
     return (weight.new_empty((), dtype=torch.float32), vals.new_empty(vals.shape, dtype=torch.float32),
-            weight.new_empty((weight.shape[1],), dtype=torch.float32), torch.empty_like(weight))
+            weight.new_empty((weight.shape[1],), dtype=torch.float32),
+            torch.empty_like(weight) if need_dw else weight.new_empty((0, weight.shape[1])))
 
 
 @torch.library.custom_op("flexsae_amd::scale_by", mutates_args=())
@@ -544,7 +569,7 @@ def scale_by(x: Tensor, grad_out: Tensor) -> Tensor:
     dev = x.device
     with torch.cuda.device(dev):
         g = _grad_scalar(grad_out, dev)
-        x = x.contiguous()
+        x = _prep(x)
         out = torch.empty_like(x)
         rc = lib.flexsae_scale(_ptr(out), _ptr(x), _DTYPES[x.dtype], x.numel(), _ptr(g), _stream())
         _lib.check(rc, "flexsae_scale")
@@ -580,7 +605,8 @@ def _is_traced(t: Tensor) -> bool:
 
 
 def _train_sliced_setup_context(ctx, inputs, output):
-    indices, weight, vals, bias, target = inputs
+    indices, weight, vals, bias, target, need_dw = inputs
+    ctx.need_dw = need_dw
     _, dvals, dbias, dW = output
     ctx.mark_non_differentiable(dvals, dbias, dW)
     ctx.leaf_dtypes = (vals.dtype, bias.dtype)
@@ -598,7 +624,9 @@ def _train_sliced_setup_context(ctx, inputs, output):
 
 def _train_sliced_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_dw):
     if grad_loss is None:
-        return None, None, None, None, None
+        return None, None, None, None, None, None
+    if ctx.needs_input_grad[1] and not ctx.need_dw:
+        raise RuntimeError("hier_train_sliced was called with need_dw=False but weight requires a gradient")
     g = grad_loss.to(torch.float32)
     vdt, bdt = ctx.leaf_dtypes
     if not ctx.dw_in_place:
@@ -615,7 +643,7 @@ def _train_sliced_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_dw):
                 with torch.no_grad():
                     _, dvals, dbias, dW = hier_train_sliced(indices, weight, vals, bias, target)
             scale_(dW, g)
-    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None
+    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None, None
 
 
 hier_train_sliced.register_autograd(_train_sliced_backward, setup_context=_train_sliced_setup_context)
@@ -662,8 +690,13 @@ def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, 
             and _train_supported(weight, indices.shape[1])):
         if _stage_fits(indices, weight):
             return hier_train(indices, weight, vals, bias, target)[0]
-        if _hier_scratch_bytes > 0:
-            return hier_train_sliced(indices, weight, vals, bias, target)[0]
+        # The slice-by-slice step rounds the unit-gradient dW to the weight dtype before the backward
+        # scales it.  fp16 cannot hold gradients of magnitude 2/(B*K*D) (they would be flushed before
+        # a loss-scaling grad_out lifts them), so fp16 weights take the separate forward + backward,
+        # which folds grad_out in before the only rounding (reference hierarchical_kernels.py:294-299
+        # scales in fp32 as well).
+        if _hier_scratch_bytes > 0 and not (weight.requires_grad and weight.dtype == torch.float16):
+            return hier_train_sliced(indices, weight, vals, bias, target, bool(weight.requires_grad))[0]
     return hier_fwd(indices, weight, vals, bias, target)[0]
 
 

@@ -70,6 +70,9 @@ enum {
   FLEXSAE_BWD_NO_DW = 32,            /* flexsae_hier_fwd_bwd only: dW is not wanted (may be     */
                                      /* NULL); the segment reductions are left out, whatever    */
                                      /* the width of the workspace, and nothing is deferred     */
+  FLEXSAE_TOPK_BWD_FP32_RESIDUAL = 256, /* flexsae_topk_bwd with bf16 weights: gather the fp32  */
+                                     /* residual instead of a bf16 copy of it (slower, and dvals */
+                                     /* then carry fp32 rounding only instead of bf16's)         */
   FLEXSAE_BWD_SKIP_EPILOGUE = 64     /* measurement aid for flexsae_hier_fwd_bwd: leave out the */
                                      /* kernels that finish loss, dvals and dbias (those        */
                                      /* outputs are then not written), so that a call with      */
@@ -256,18 +259,23 @@ int flexsae_hier_import_pair_list(const flexsae_shape *shape, const uint32_t *be
  * replaces: aggregate_gradient_for_embedding_kernel and its launch, plus the autograd of
  *           the eager loss tail that produces `gradient` and the bias gradient
  *           (topk_kernels.py:97-137, 165-184, 220-223)
- * in : begin/map from flexsae_csr_build; resid from flexsae_topk_fwd; grad_out device scalar.
+ * in : begin/map from flexsae_csr_build; resid from flexsae_topk_fwd; grad_out device scalar;
+ *      indices[B,K] (may be NULL): when given, a pair whose index lies outside [0, F) counts with a
+ *      value of zero, as it did in the forward (the pair list files it under latent 0), so dW, dvals
+ *      and dbias are the gradients of the loss the forward returned; NULL skips that test.
  * out: dW[F,D] written once in `dW_dtype` (every row, zeros for unused latents);
  *      dvals[B,K] fp32, every element written once (per-tile shares added in tile order);
  *      dbias[D] fp32 (column sums in a fixed order).  All three are bit-reproducible;
- *      `flags` is accepted for symmetry and ignored (nothing needs a zero-fill).
+ *      nothing needs a zero-fill (FLEXSAE_BWD_OUTPUTS_PREZEROED is accepted and ignored).
  * With bf16 weights the residual rows are gathered from a bf16 copy made in the workspace: the
  * reference's backward likewise receives the residual gradient in the weight dtype
- * (topk_kernels.py:52 makes the bag output weight-typed, so autograd casts its gradient).
+ * (topk_kernels.py:52 makes the bag output weight-typed, so autograd casts its gradient).  That
+ * rounding shows in dvals (about 4e-3 normwise instead of 1e-6); FLEXSAE_TOPK_BWD_FP32_RESIDUAL in
+ * `flags` gathers the fp32 residual instead (twice the cache footprint, slower).
  * Limit: B*D*4 bytes < 4 GiB (FLEXSAE_ERR_UNSUPPORTED beyond), the gathers use 32-bit offsets.
  */
 int flexsae_topk_bwd(const flexsae_shape *shape, const uint32_t *begin, const uint32_t *map,
-                     const void *weight, const void *vals, const float *resid,
+                     const int64_t *indices, const void *weight, const void *vals, const float *resid,
                      const float *grad_out, void *dW, int dW_dtype, float *dvals, float *dbias,
                      void *workspace, size_t workspace_bytes, int flags, void *stream);
 

@@ -58,16 +58,20 @@ def hier_backward(indices, weight, vals, resid, grad_out, flag=None, slice_cols=
     return rc, dW, dv, db
 
 
-def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_dtype=torch.float32, flags=0):
-    """Fused forward+backward for a unit upstream gradient -> (rc, loss, dW, dvals, dbias)."""
+def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_dtype=torch.float32, flags=0,
+               alloc_dw=True):
+    """Fused forward+backward for a unit upstream gradient -> (rc, loss, dW, dvals, dbias);
+    ``alloc_dw=False`` passes a null dW (for FLEXSAE_BWD_NO_DW)."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
     dev = weight.device
     loss = torch.full((1,), float("nan"), dtype=torch.float32, device=dev)
-    dW = torch.full((sh.F, sh.D), float("nan"), dtype=dw_dtype, device=dev)
+    dW = torch.full((sh.F, sh.D), float("nan"), dtype=dw_dtype, device=dev) if alloc_dw else None
     dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
     db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
-    nbytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+    # slices of whole training tiles where the entry point supports the shape
+    nbytes = (lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+              or lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols))
     ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
     rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(bias), ptr(target),
                                   ptr(loss), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, flags,
@@ -117,7 +121,7 @@ def widen_u32(t):
     return t.to(torch.int64) & 0xFFFFFFFF
 
 
-def topk_backward(indices, weight, vals, resid, grad_out, dw_dtype=None, slice_cols=0):
+def topk_backward(indices, weight, vals, resid, grad_out, dw_dtype=None, slice_cols=0, flags=0, pass_indices=True):
     """-> (rc, dW in dw_dtype, dvals fp32, dbias fp32); builds the pair list first."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals)
@@ -132,8 +136,9 @@ def topk_backward(indices, weight, vals, resid, grad_out, dw_dtype=None, slice_c
     g = torch.tensor([grad_out], dtype=torch.float32, device=dev)
     nbytes = lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    rc = lib.flexsae_topk_bwd(ctypes.byref(sh), ptr(begin), ptr(mp), ptr(weight), ptr(vals), ptr(resid),
-                              ptr(g), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, 0, stream())
+    rc = lib.flexsae_topk_bwd(ctypes.byref(sh), ptr(begin), ptr(mp), ptr(indices if pass_indices else None),
+                              ptr(weight), ptr(vals), ptr(resid),
+                              ptr(g), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, flags, stream())
     return rc, dW, dv, db
 
 

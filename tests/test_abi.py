@@ -120,11 +120,14 @@ def test_backward_and_csr_reject_bad_arguments():
     assert lib.flexsae_csr_build(NULL, 4, 8, 16, FAKE, FAKE, FAKE, 1 << 20, NULL, NULL) == _lib.ERR_INVALID_ARGUMENT
     assert lib.flexsae_csr_build(FAKE, 4, 8, 16, FAKE, FAKE, FAKE, 4, NULL, NULL) == _lib.ERR_WORKSPACE
     assert lib.flexsae_csr_build(FAKE, 1 << 20, 1 << 12, 16, FAKE, FAKE, FAKE, 1 << 20, NULL, NULL) == _lib.ERR_UNSUPPORTED
-    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 9, FAKE, FAKE, FAKE,
+    # (shape, begin, map, indices or NULL, weight, vals, resid, grad_out, dW, dW_dtype, dvals, dbias, ws, bytes, flags, stream)
+    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, NULL, FAKE, FAKE, FAKE, FAKE, FAKE, 9, FAKE, FAKE, FAKE,
                                 1 << 20, 0, NULL) == _lib.ERR_INVALID_ARGUMENT
-    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, NULL, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, FAKE,
+    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, NULL, NULL, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, FAKE,
                                 1 << 20, 0, NULL) == _lib.ERR_INVALID_ARGUMENT
-    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, NULL,
+    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, ctypes.c_void_p(0x10004), FAKE, FAKE, FAKE, FAKE, FAKE, 0,
+                                FAKE, FAKE, FAKE, 1 << 20, 0, NULL) == _lib.ERR_ALIGNMENT
+    assert lib.flexsae_topk_bwd(ctypes.byref(sh), FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 0, FAKE, FAKE, NULL,
                                 1 << 20, 0, NULL) == _lib.ERR_WORKSPACE
     assert lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh), 0) >= 64 * 4
     assert (lib.flexsae_topk_bwd_workspace_bytes(ctypes.byref(sh), 1 << 30)

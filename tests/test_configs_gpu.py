@@ -65,19 +65,34 @@ def _run(mode, idx, W, v, b, t, grad_out=1.0):
     return loss.detach(), Wp.grad, vp.grad, bp.grad
 
 
+def _elementwise(name, got, ref, tol):
+    """The parity bar for one gradient tensor: ||got - ref|| <= tol ||ref|| and, element by element,
+    |got - ref| <= tol |ref| + tol max|ref| (float64, in row blocks to bound the memory)."""
+    got2, ref2 = got.reshape(-1, got.shape[-1]), ref.reshape(-1, ref.shape[-1])
+    ref_max = float(ref2.abs().max())
+    num = den = 0.0
+    worst = -1.0
+    blk = max(1, (1 << 24) // ref2.shape[1])
+    for r0 in range(0, ref2.shape[0], blk):
+        g, r = got2[r0:r0 + blk].double(), ref2[r0:r0 + blk].double()
+        diff = (g - r).abs()
+        num += float((diff ** 2).sum())
+        den += float((r ** 2).sum())
+        worst = max(worst, float((diff - tol * r.abs()).max()) - tol * ref_max)
+    assert num ** 0.5 <= tol * den ** 0.5, f"{name}: rel err {(num / den) ** 0.5:.3e} > {tol}"
+    assert worst <= 0, f"{name}: an element misses rtol={tol}, atol={tol}*max|ref| by {worst:.3e}"
+
+
 def _full_compare(mode, args, dtype, grad_out, tol_loss, tol_grad):
     idx, W, v, b, t = args
     loss, dW, dv, db = _run(mode, *args, grad_out=grad_out)
     cpu = [x.cpu() for x in args]
     L, rW, rv, rb = oracle.loss_grads(MODES[mode], *cpu, grad_out=grad_out, dw_float32=True)
     assert abs(loss.item() - L) <= tol_loss * abs(L), (loss.item(), L)
-    assert rel_err(dv.float().cpu(), rv) <= tol_grad
-    assert rel_err(db.float().cpu(), rb) <= tol_grad
-    # dW: normwise error in float64 on the GPU (the matrices are large)
-    rWd = torch.from_numpy(rW).to(DEV)
-    num = (dW.double() - rWd.double()).norm().item()
-    den = rWd.double().norm().item()
-    assert num / den <= tol_grad, f"dW rel err {num / den:.3e}"
+    _elementwise("dvals", dv.cpu(), torch.from_numpy(rv), tol_grad)
+    _elementwise("dbias", db.cpu(), torch.from_numpy(rb), tol_grad)
+    # dW on the GPU (the matrices are large): normwise and element by element
+    _elementwise("dW", dW, torch.from_numpy(rW).to(DEV), tol_grad)
     touched = torch.zeros(W.shape[0], dtype=torch.bool, device=DEV)
     touched[idx.flatten()] = True
     assert torch.count_nonzero(dW[~touched]) == 0
@@ -90,7 +105,8 @@ def test_config1_fp32_small(mode):
     _full_compare(mode, args, torch.float32, 1.0, 1e-5, 1e-4)
 
 
-@pytest.mark.parametrize("mode,K", [("hier", 128), ("topk", 128), ("hier", 32), ("hier", 64)])
+@pytest.mark.parametrize("mode,K", [("hier", 128), ("topk", 128), ("hier", 32), ("hier", 64), ("topk", 32),
+                                    ("topk", 64)])
 def test_config2_bf16(mode, K):
     print("[case] config2", mode, K, flush=True)
     args = _gen(4096, K, 65536, 2304, torch.bfloat16, "unique")
@@ -114,9 +130,9 @@ def _subset_parity(mode, args, rows, tol_loss, tol_grad):
     L, rW, rv, rb = oracle.loss_grads(MODES[mode], inv.cpu(), Wc, sub[2].cpu(), b.cpu(), sub[4].cpu(),
                                       dw_float32=True)
     assert abs(loss.item() - L) <= tol_loss * abs(L), (loss.item(), L)
-    assert rel_err(dv.float().cpu(), rv) <= tol_grad
-    assert rel_err(db.float().cpu(), rb) <= tol_grad
-    assert rel_err(dW[uniq].float().cpu(), rW) <= tol_grad
+    _elementwise("dvals", dv.cpu(), torch.from_numpy(rv), tol_grad)
+    _elementwise("dbias", db.cpu(), torch.from_numpy(rb), tol_grad)
+    _elementwise("dW", dW[uniq].cpu(), torch.from_numpy(rW), tol_grad)
     mask = torch.ones(W.shape[0], dtype=torch.bool, device=DEV)
     mask[uniq] = False
     assert torch.count_nonzero(dW[mask]) == 0
@@ -158,7 +174,7 @@ def test_config4_bf16_zipf():
     args = _gen(8192, 64, 262144, 4096, torch.bfloat16, "zipf", w_std=0.02)
     counts = torch.bincount(args[0].flatten(), minlength=262144)
     assert counts.max().item() > 4096  # the hottest latent is in most rows
-    _subset_parity("hier", args, 512, 1e-2, 1e-2)
+    _subset_parity("hier", args, 2048, 1e-2, 1e-2)
     _additivity_and_conservation("hier", args, 4, 1e-2)
 
 
@@ -166,7 +182,7 @@ def test_config4_bf16_zipf():
 def test_config5_bf16_large(mode):
     print("[case] config5", mode, flush=True)
     args = _gen(16384, 128, 524288, 8192, torch.bfloat16, "unique", w_std=0.02)
-    _subset_parity(mode, args, 256, 1e-2, 1e-2)
+    _subset_parity(mode, args, 1024, 1e-2, 1e-2)
     _additivity_and_conservation(mode, args, 2, 1e-2)
     del args
     torch.cuda.empty_cache()

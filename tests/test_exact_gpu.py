@@ -1,0 +1,196 @@
+"""Bit-exact checks of every gathering / scattering kernel (the north star asks for bit-exact
+indices and gather addressing; reference kernels address with int64 throughout,
+hierarchical_kernels.py:34-42,115-123 and topk_kernels.py:29-30).
+
+Inputs are small integers and B*K*D (or B*D) is a power of two, so every quantity the kernels form
+is an integer multiple of a power of two that fits the fp32 mantissa: sums are exact in any order,
+and a single row read from, or a single contribution written to, a wrong address changes the result.
+Expected values come from the definitions in float64.
+"""
+import pytest
+import torch
+
+import abi
+from flexsae_amd import _lib
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _announce(*what):
+    print("[case]", *what, flush=True)
+
+
+def _coded(rows, cols, modulus):
+    """W[f, d] = a small integer code of (f, d): a wrong row or column shows."""
+    f = torch.arange(rows, dtype=torch.int64).unsqueeze(1)
+    d = torch.arange(cols, dtype=torch.int64).unsqueeze(0)
+    return (((f * 2654435761 + d * 40503) >> 7) % modulus).double()
+
+
+def _hier_exact(idx, W, v, bias, target):
+    """Loss and gradients of the hierarchical loss from its definition, float64 (reference
+    hierarchical_kernels.py:312-323 and the reverse walk at 135-167)."""
+    B, K = idx.shape
+    F, D = W.shape
+    e = bias - target[:, None, :] + (W[idx] * v[..., None]).cumsum(1)
+    count = B * K * D
+    loss = (e ** 2).sum() / count
+    S = (2.0 / count * e).flip(1).cumsum(1).flip(1)
+    dvals = (W[idx] * S).sum(-1)
+    dbias = S[:, 0, :].sum(0)
+    dW = torch.zeros(F, D, dtype=torch.float64).index_add_(0, idx.flatten(), (v[..., None] * S).reshape(-1, D))
+    return loss, dW, dvals, dbias, e[:, -1, :]
+
+
+# (B, K, F, D, dtype, weight modulus): B*K*D is a power of two everywhere.
+#  fp32 K<=64 : two columns per lane;  fp32 K>64 : one column per lane, two index chunks per row
+#  bf16       : contributions are staged in bf16: dW is compared exactly where S stays below 2^8
+#               (short rows), to 1e-2 for the 128-step rows (dvals and dbias stay exact: fp32)
+#  F tiny     : latents with more than 64 pairs (chunked reduction + finalize)
+HIER_CASES = [
+    (32, 4, 4096, 64, torch.float32, 8),
+    (8, 64, 1 << 14, 256, torch.float32, 2),
+    (8, 128, 1 << 15, 64, torch.float32, 2),
+    (16, 32, 4, 128, torch.float32, 2),
+    (64, 2, 1 << 13, 128, torch.bfloat16, 4),
+    (32, 4, 1 << 13, 256, torch.bfloat16, 2),
+    (4, 128, 1 << 16, 128, torch.bfloat16, 2),
+]
+
+
+def _make_hier_case(B, K, F, D, dtype, modulus, seed):
+    g = torch.Generator().manual_seed(seed)
+    W = _coded(F, D, modulus)
+    if F >= B * K * 4:
+        idx = torch.randperm(F, generator=g)[: B * K].reshape(B, K)  # no latent twice: bf16 dW stays exact
+    else:
+        idx = torch.randint(0, F, (B, K), generator=g)
+    v = torch.ones(B, K, dtype=torch.float64)
+    bias = torch.zeros(D, dtype=torch.float64)
+    target = torch.zeros(B, D, dtype=torch.float64)
+    return idx, W, v, bias, target
+
+
+@pytest.mark.parametrize("case", HIER_CASES, ids=lambda c: f"B{c[0]}K{c[1]}F{c[2]}D{c[3]}{str(c[4])[6:]}")
+@pytest.mark.parametrize("slices", ["narrow", "wide"])
+def test_hier_training_step_addressing_is_exact(case, slices):
+    """flexsae_hier_fwd_bwd: the row gathers of the training-step kernel (per-row buffer descriptors),
+    its contribution stores (slot addressing) and the segment reduction that reads them back."""
+    B, K, F, D, dtype, modulus = case
+    _announce("exact train", case, slices)
+    idx, W, v, bias, target = _make_hier_case(B, K, F, D, dtype, modulus, seed=B + K)
+    loss_x, dW_x, dv_x, db_x, _ = _hier_exact(idx, W, v, bias, target)
+    assert dW_x.abs().max() < (1 << 24) * 2.0 / (B * K * D)
+    # bf16 weights: staged contributions and dW entries are exact in bf16 only below 2^8 units
+    exact_dw = dtype != torch.bfloat16 or dW_x.abs().max() * (B * K * D) / 2.0 < 256
+    assert exact_dw or K == 128
+    dev_args = [idx.to(DEV)] + [x.to(dtype).to(DEV) for x in (W, v, bias, target)]
+    rc, loss, dW, dv, db = abi.hier_train(*dev_args, slice_cols=(0 if slices == "narrow" else 1 << 20),
+                                          dw_dtype=dtype)
+    torch.cuda.synchronize()
+    assert rc == 0, _lib.status_string(rc)
+    assert torch.equal(dv.double().cpu(), dv_x)
+    assert torch.equal(db.double().cpu(), db_x)
+    if exact_dw:
+        assert torch.equal(dW.double().cpu(), dW_x)
+    else:
+        assert (dW.double().cpu() - dW_x).norm() <= 1e-2 * dW_x.norm()
+    if float(loss_x) * (B * K * D) < (1 << 24):
+        assert loss.double().item() == float(loss_x)
+    else:
+        assert abs(loss.item() - float(loss_x)) <= 1e-6 * float(loss_x)
+
+
+@pytest.mark.parametrize("case", HIER_CASES[:4] + HIER_CASES[4:6],
+                         ids=lambda c: f"B{c[0]}K{c[1]}F{c[2]}D{c[3]}{str(c[4])[6:]}")
+def test_hier_sweep_addressing_is_exact(case):
+    """flexsae_hier_fwd + flexsae_hier_bwd: the gathers of the forward kernel and of the reverse
+    sweep kernel, and the sweep's contribution stores."""
+    B, K, F, D, dtype, modulus = case
+    _announce("exact sweep", case)
+    idx, W, v, bias, target = _make_hier_case(B, K, F, D, dtype, modulus, seed=B + K)
+    loss_x, dW_x, dv_x, db_x, resid_x = _hier_exact(idx, W, v, bias, target)
+    dev_args = [idx.to(DEV)] + [x.to(dtype).to(DEV) for x in (W, v, bias, target)]
+    rc, loss, resid = abi.forward("hier", *dev_args)
+    assert rc == 0
+    assert torch.equal(resid.double().cpu(), resid_x)
+    rc, dW, dv, db = abi.hier_backward(dev_args[0], dev_args[1], dev_args[2], resid, 1.0, dw_dtype=dtype)
+    torch.cuda.synchronize()
+    assert rc == 0, _lib.status_string(rc)
+    assert torch.equal(dv.double().cpu(), dv_x)
+    assert torch.equal(db.double().cpu(), db_x)
+    assert torch.equal(dW.double().cpu(), dW_x)
+
+
+@pytest.mark.parametrize("dtype,fp32_residual", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)],
+                         ids=["fp32", "bf16-resid16", "bf16-resid32"])
+@pytest.mark.parametrize("shape", [(64, 8, 4096, 512), (32, 16, 6, 1024), (16, 4, 1 << 15, 256)])
+def test_topk_backward_addressing_is_exact(shape, dtype, fp32_residual):
+    """flexsae_topk_bwd: the residual-row gathers (32-bit offsets through a buffer descriptor), the
+    weight-row loads and the dW / dvals stores, from an integer-coded residual.
+    dW[f] = scale * sum of the residual rows of f's pairs, dvals[p] = scale * <resid[b], W[f]>."""
+    B, K, F, D = shape
+    _announce("exact topk bwd", shape, dtype, fp32_residual)
+    g = torch.Generator().manual_seed(B * K)
+    idx = torch.randint(0, F, (B, K), generator=g)
+    resid = _coded(B, D, 4 if F > 8 else 2)      # sums of a latent's rows stay exact in bf16 as well
+    W = _coded(F, D, 2) if F > 8 else _coded(F, D, 4)
+    v = torch.ones(B, K, dtype=torch.float64)
+    scale = 2.0 / (B * D)                        # a power of two
+    dW_x = torch.zeros(F, D, dtype=torch.float64).index_add_(
+        0, idx.flatten(), (scale * resid)[:, None, :].expand(B, K, D).reshape(-1, D))
+    dv_x = scale * (resid[:, None, :] * W[idx]).sum(-1)
+    db_x = scale * resid.sum(0)
+    if dtype == torch.bfloat16:
+        assert (dW_x / scale).abs().max() < 256  # exact in the bf16 gradient
+    rc, dW, dv, db = abi.topk_backward(idx.to(DEV), W.to(dtype).to(DEV), v.to(dtype).to(DEV),
+                                       resid.float().to(DEV), 1.0, dw_dtype=dtype,
+                                       flags=_lib.TOPK_BWD_FP32_RESIDUAL if fp32_residual else 0)
+    torch.cuda.synchronize()
+    assert rc == 0, _lib.status_string(rc)
+    assert torch.equal(dv.double().cpu(), dv_x)
+    assert torch.equal(db.double().cpu(), db_x)
+    assert torch.equal(dW.double().cpu(), dW_x)
+
+
+def test_rows_beyond_four_gib_are_addressed_exactly():
+    """The weight matrix of the largest configuration (F=524288, D=8192, bf16: 8.6 GB): rows whose
+    byte offset lies beyond 2^32 (up to the last row, just below 2^33) are gathered exactly by the
+    forward kernel and by the training-step kernel.  W[f, d] is a 2-bit hash of (f, d), generated on the device."""
+    F, D, B, K = 524288, 8192, 64, 8
+    _announce("exact >4GiB", F, D)
+    W = torch.empty(F, D, dtype=torch.bfloat16, device=DEV)
+    d = torch.arange(D, device=DEV, dtype=torch.int64).unsqueeze(0) * 40503
+    for f0 in range(0, F, 8192):
+        f = torch.arange(f0, f0 + 8192, device=DEV, dtype=torch.int64).unsqueeze(1) * 2654435761
+        W[f0:f0 + 8192] = (((f + d) >> 7) % 4).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(5)
+    idx = torch.randint(0, F, (B, K), generator=g)
+    # the rows on either side of the 2^32-byte offset, the last rows (just below 2^33 bytes), row 0
+    row_bytes = D * 2
+    special = [(1 << 32) // row_bytes - 1, (1 << 32) // row_bytes, F - 2, F - 1, 0, F // 2 + 1,
+               3 * (F // 4) + 5, (3 << 31) // row_bytes]
+    idx[0] = torch.tensor(special)
+    assert 0 <= idx.min().item() and idx.max().item() == F - 1 and (F - 1) * row_bytes > (1 << 32)
+    dd = torch.arange(D, dtype=torch.int64) * 40503
+    expect = (((idx.unsqueeze(-1) * 2654435761 + dd) >> 7) % 4).double()   # [B, K, D] row pieces
+    resid_x = expect.sum(1)
+    v = torch.ones(B, K, dtype=torch.bfloat16, device=DEV)
+    bias = torch.zeros(D, dtype=torch.bfloat16, device=DEV)
+    target = torch.zeros(B, D, dtype=torch.bfloat16, device=DEV)
+    for mode in ("hier", "topk"):
+        rc, loss, resid = abi.forward(mode, idx.to(DEV), W, v, bias, target)
+        torch.cuda.synchronize()
+        assert rc == 0
+        assert torch.equal(resid.double().cpu(), resid_x), mode
+    # training-step kernel (no dW: it would be another 8.6 GB): dvals and dbias are exact sums
+    e = expect.cumsum(1)
+    S = (2.0 / (B * K * D) * e).flip(1).cumsum(1).flip(1)   # B*K*D = 2^22
+    dv_x = (expect * S).sum(-1)
+    db_x = S[:, 0, :].sum(0)
+    rc, loss, _, dv, db = abi.hier_train(idx.to(DEV), W, v, bias, target, flags=_lib.BWD_NO_DW, alloc_dw=False)
+    torch.cuda.synchronize()
+    assert rc == 0, _lib.status_string(rc)
+    assert torch.equal(dv.double().cpu(), dv_x)
+    assert torch.equal(db.double().cpu(), db_x)

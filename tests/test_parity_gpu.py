@@ -46,6 +46,27 @@ def _run_op(mode, args_cpu, grad_out):
     return loss, W.grad, v.grad, b.grad
 
 
+def check_gradient(name, got, ref, dtype, tol):
+    """The parity bar for one gradient tensor against the oracle's float64 result:
+    normwise ||got - ref|| <= tol * ||ref||, and element by element
+    |got - ref| <= tol * |ref| + tol * max|ref|.
+    fp32 and bf16 leaves get exactly that.  fp16 leaves get, on top, what rounding the exact
+    gradient to fp16 costs by itself: gradients of magnitude 2/(B*K*D) are subnormal in fp16
+    (spacing 6e-8), so their rounding error alone can exceed any relative tolerance."""
+    ref_t = torch.as_tensor(ref, dtype=torch.float64)
+    got_t = got.detach().double().cpu()
+    err = rel_err(got_t, ref_t)
+    quant_rel, quant_abs = 0.0, 0.0
+    if dtype == torch.float16:
+        rounded = ref_t.to(dtype).double()
+        quant_rel = 1.5 * rel_err(rounded, ref_t)
+        quant_abs = 1.5 * float((rounded - ref_t).abs().max())
+    assert err <= tol + quant_rel, f"{name}: rel err {err:.3e} > {tol} (+ {quant_rel:.3e})"
+    bound = tol * ref_t.abs() + tol * float(ref_t.abs().max()) + quant_abs
+    worst = float(((got_t - ref_t).abs() - bound).max())
+    assert worst <= 0, f"{name}: an element misses rtol={tol}, atol={tol}*max|ref| by {worst:.3e}"
+
+
 def _check_against_oracle(mode, args_cpu, dtype, grad_out, got, ref_tols=True):
     loss, dW, dv, db = got
     L, rW, rv, rb = oracle.loss_grads(MODES[mode], *args_cpu, grad_out=grad_out)
@@ -54,11 +75,7 @@ def _check_against_oracle(mode, args_cpu, dtype, grad_out, got, ref_tols=True):
     assert abs(loss.item() - L) <= tol_loss * abs(L), (loss.item(), L)
     assert dW.dtype == dtype and dv.dtype == dtype and db.dtype == dtype
     for name, g, r in (("dW", dW, rW), ("dvals", dv, rv), ("dbias", db, rb)):
-        err = rel_err(g.float().cpu(), r)
-        # what rounding the exact gradient to the leaf dtype costs by itself (fp16 gradients of
-        # magnitude 2/(B*K*D) are subnormal, so this can exceed the arithmetic tolerance)
-        quant = rel_err(torch.from_numpy(r).to(dtype).double(), r)
-        assert err <= tol_grad + 1.5 * quant, f"{name}: rel err {err:.3e} > {tol_grad} + 1.5*{quant:.3e}"
+        check_gradient(name, g, r, dtype, tol_grad)
     if ref_tols:
         tols = DTYPE_TO_TOLS[dtype]
         torch.testing.assert_close(loss.cpu(), torch.tensor(L, dtype=torch.float32), **tols)
@@ -468,6 +485,109 @@ def test_out_of_range_index_is_flagged_not_followed(mode):
     with pytest.raises(IndexError):
         flex.check_index_flag()
     flex.check_index_flag()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("mode,path", [("hier", "default"), ("hier", "staged"), ("hier", "unfused"), ("topk", "default")])
+def test_out_of_range_index_gradients(mode, path, dtype):
+    """The gradients with out-of-range indices are those of the loss the forward returned: the
+    offending pairs count as (latent 0, value 0) in dW, dvals and dbias of both losses, on every
+    path (one of the pairs sits in a latent-0 group that also has regular pairs)."""
+    B, K, F, D = 24, 16, 40, 256
+    idx, W, v, b, t = make_inputs(B, K, F, D, dtype=dtype, seed=8)
+    idx[3, 2] = F
+    idx[5, 0] = -1
+    idx[7, 9] = 1 << 40
+    idx[2, 1] = 0           # a regular pair of latent 0
+    idx2, v2 = idx.clone(), v.clone()
+    for (r, c) in ((3, 2), (5, 0), (7, 9)):
+        idx2[r, c] = 0
+        v2[r, c] = 0
+    flex.set_fused_training(path != "unfused")
+    flex.set_hier_stage_bytes(STAGE_ALL if path == "staged" else None)
+    try:
+        got = _run_op(mode, (idx, W, v, b, t), 1.3)
+    finally:
+        flex.set_fused_training(True)
+        flex.set_hier_stage_bytes(None)
+    try:
+        flex.check_index_flag()
+    except IndexError:
+        pass
+    _check_against_oracle(mode, (idx2, W, v2, b, t), dtype, 1.3, got, ref_tols=False)
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_fp16_weights_with_a_loss_scaling_upstream_gradient(mode):
+    """fp16 leaves and grad_out = 2^16 (what a gradient scaler passes): the unit gradients, about
+    2/(B*K*D), are far below fp16's range and must not be rounded to fp16 before the upstream
+    gradient lifts them (the reference scales its fp32 gradients first, reference
+    hierarchical_kernels.py:294-299)."""
+    B, K, F, D = 64, 32, 224, 1024
+    args = make_inputs(B, K, F, D, dtype=torch.float16, seed=21)
+    grad_out = 65536.0
+    got = _run_op(mode, args, grad_out)
+    L, rW, rv, rb = oracle.loss_grads(MODES[mode], *args, grad_out=grad_out)
+    # the scaled gradients are normal fp16 numbers: the plain fp16 bar applies, without any allowance
+    assert float(np.abs(rW).max()) > 1e-4
+    for name, g, r in (("dW", got[1], rW), ("dvals", got[2], rv), ("dbias", got[3], rb)):
+        err = rel_err(g.float().cpu(), r)
+        assert err <= 1e-3, f"{name}: {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_storage_offset_views(mode, dtype):
+    """Contiguous tensors that start at an odd element of a larger buffer (a bias cut out of a flat
+    parameter vector, a weight view): forward and backward work as in the reference, which
+    addresses element-wise."""
+    B, K, F, D = 16, 8, 40, 260
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=31)
+    idx, W, v, b, t = _to_dev(args)
+
+    def off_by_one(x):
+        flat = torch.empty(x.numel() + 1, dtype=x.dtype, device=DEV)
+        view = flat[1:].view(x.shape)
+        view.copy_(x)
+        assert view.is_contiguous() and view.data_ptr() % 16 != 0
+        return view.requires_grad_()
+
+    Wv, vv, bv = off_by_one(W), off_by_one(v), off_by_one(b)
+    tv = off_by_one(t).detach()
+    loss = FUSED[mode](idx, Wv, vv, bv, tv)
+    loss.backward(torch.tensor(0.9, device=DEV))
+    torch.cuda.synchronize()
+    _check_against_oracle(mode, args, dtype, 0.9, (loss, Wv.grad, vv.grad, bv.grad), ref_tols=False)
+    with torch.no_grad():
+        loss2 = FUSED[mode](idx, Wv, vv, bv, tv)
+    assert abs(loss2.item() - loss.item()) <= 1e-6 * abs(loss.item())
+
+
+def test_topk_residual_precision_switch():
+    """bf16 weights: the TopK backward gathers a bf16 copy of the residual by default (as the
+    reference's backward receives it, reference topk_kernels.py:52); with the switch off it gathers
+    the fp32 residual and dvals carry fp32 rounding only.  Both meet the bf16 bar."""
+    B, K, F, D = 96, 32, 320, 1536
+    args = make_inputs(B, K, F, D, dtype=torch.bfloat16, seed=23)
+    L, rW, rv, rb = oracle.loss_grads(oracle.TOPK, *args, grad_out=0.7)
+    idx, W, v, b, t = _to_dev(args)
+    rc, loss, resid = abi.forward("topk", idx, W, v, b, t)
+    errs = {}
+    for name, flags in (("bf16", 0), ("fp32", abi._lib.TOPK_BWD_FP32_RESIDUAL)):
+        rc, dW, dv, db = abi.topk_backward(idx, W, v, resid, 0.7, dw_dtype=torch.float32, flags=flags)
+        torch.cuda.synchronize()
+        assert rc == 0
+        errs[name] = (rel_err(dW.cpu(), rW), rel_err(dv.cpu(), rv), rel_err(db.cpu(), rb))
+        print("[topk residual]", name, "dW %.2e dvals %.2e dbias %.2e" % errs[name], flush=True)
+    assert errs["bf16"][0] < 1e-2 and errs["bf16"][1] < 1e-2
+    assert errs["fp32"][0] < 1e-4 and errs["fp32"][1] < 1e-4 and errs["fp32"][2] < 1e-4
+    # the python switch reaches the same two variants
+    flex.set_topk_residual_bf16(False)
+    try:
+        got = _run_op("topk", args, 0.7)
+    finally:
+        flex.set_topk_residual_bf16(True)
+    _check_against_oracle("topk", args, torch.bfloat16, 0.7, got, ref_tols=False)
 
 
 def test_topk_target_gradient():
