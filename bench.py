@@ -9,7 +9,9 @@ the latency ratio, the two dominant kernels are timed alone with HIP events for 
 object, and a torch restatement of the reference's eager path is timed on the host cores on a
 bounded row sample as the CPU baseline.
 
-Prints ONE JSON line on stdout.  ``python bench.py --gpus 1 --steps 20 --warmup 5``.
+Prints ONE JSON line on stdout.  ``python bench.py`` = ``--gpus 1 --steps 100 --warmup 5``, the
+protocol of the reference's timing script (5 warm-up + 100 timed iterations, events around
+``loss = f(...); loss.backward()``, mean and standard deviation; reference example.py:30-36, 70-101).
 """
 import argparse
 import ctypes
@@ -35,7 +37,7 @@ WORKLOADS = {
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_k128", choices=sorted(WORKLOADS))
     ap.add_argument("--shape", default="", help="override B,K,F,D of the workload (tuning aid)")
@@ -47,35 +49,42 @@ def parse_args():
 
 
 def make_inputs(torch, B, K, F, D, dtype, dist, w_std, device):
-    """Seeded synthetic inputs, generated on the device (indices/vals/weight/bias/target)."""
-    g = torch.Generator(device=device).manual_seed(1234)
+    """Seeded synthetic inputs in the order indices, vals, weight, bias, target (seed 1234, the
+    reference's test seed, reference tests/test_setup.py:3).  Workloads whose weight matrix has at
+    most 2^28 elements are generated with the CPU generator and moved to the device, so the CPU
+    baseline and the GPU see tensors anyone can regenerate; larger ones are generated on the device
+    (the CPU legs still get the same tensors, copied back).  Returns (tensors, where)."""
+    on_cpu = F * D <= (1 << 28)
+    gdev = "cpu" if on_cpu else device
+    g = torch.Generator(device=gdev).manual_seed(1234)
     if dist == "randint":
-        idx = torch.randint(0, F, (B, K), generator=g, device=device, dtype=torch.long)
+        idx = torch.randint(0, F, (B, K), generator=g, device=gdev, dtype=torch.long)
     else:
-        idx = torch.empty(B, K, dtype=torch.long, device=device)
-        step = max(1, (1 << 26) // F)
+        idx = torch.empty(B, K, dtype=torch.long, device=gdev)
+        step = max(1, ((1 << 24) if on_cpu else (1 << 26)) // F)
         if dist == "zipf":
-            logp = -1.1 * torch.log(torch.arange(1, F + 1, dtype=torch.float32, device=device))
-            perm = torch.randperm(F, generator=g, device=device)
+            logp = -1.1 * torch.log(torch.arange(1, F + 1, dtype=torch.float32, device=gdev))
+            perm = torch.randperm(F, generator=g, device=gdev)
         for b0 in range(0, B, step):
             n = min(step, B - b0)
-            u = torch.rand(n, F, generator=g, device=device)
+            u = torch.rand(n, F, generator=g, device=gdev)
             if dist == "zipf":
                 key = logp - torch.log(-torch.log(u.clamp_(1e-30, 1 - 1e-7)))
                 idx[b0:b0 + n] = perm[key.topk(K, dim=1).indices]
             else:
                 idx[b0:b0 + n] = u.topk(K, dim=1).indices
-    vals = torch.randn(B, K, generator=g, device=device).abs()
+    vals = torch.randn(B, K, generator=g, device=gdev).abs()
     if dist == "zipf":
         vals = vals.sort(dim=1, descending=True).values
-    weight = torch.empty(F, D, dtype=dtype, device=device)
+    weight = torch.empty(F, D, dtype=dtype, device=gdev)
     rows = max(1, (1 << 27) // D)
     for f0 in range(0, F, rows):
         n = min(rows, F - f0)
-        weight[f0:f0 + n] = (torch.randn(n, D, generator=g, device=device) * w_std).to(dtype)
-    bias = torch.randn(D, generator=g, device=device).to(dtype)
-    target = torch.randn(B, D, generator=g, device=device).to(dtype)
-    return idx, weight, vals.to(dtype), bias, target
+        weight[f0:f0 + n] = (torch.randn(n, D, generator=g, device=gdev) * w_std).to(dtype)
+    bias = torch.randn(D, generator=g, device=gdev).to(dtype)
+    target = torch.randn(B, D, generator=g, device=gdev).to(dtype)
+    out = tuple(x.to(device) for x in (idx, weight, vals.to(dtype), bias, target))
+    return out, ("cpu generator" if on_cpu else "device generator")
 
 
 def algorithmic_bytes(B, K, F, D, sw, st, sv):
@@ -96,14 +105,24 @@ def algorithmic_bytes(B, K, F, D, sw, st, sv):
 
 
 def time_steps(torch, fn, steps, warmup):
+    """W untimed steps, then exactly K steps between two synchronisations (wall clock); every timed
+    step is also bracketed by a pair of events for the spread.  Returns (ms per step by the wall
+    clock, mean of the per-step event times, their standard deviation)."""
     for _ in range(warmup):
         fn()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for e0, e1 in events:
+        e0.record()
         fn()
+        e1.record()
     torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps * 1e3
+    wall = (time.perf_counter() - t0) / steps * 1e3
+    per = [e0.elapsed_time(e1) for e0, e1 in events]
+    mean = sum(per) / len(per)
+    std = (sum((x - mean) ** 2 for x in per) / max(1, len(per) - 1)) ** 0.5
+    return wall, mean, std
 
 
 def time_kernel_events(torch, prepare, launch, steps, warmup):
@@ -132,8 +151,13 @@ def cpu_baseline(torch, mode_name, inputs, full_B, rows=0):
     the dense weight-gradient buffer, which the sample pays in full)."""
     import oracle
 
-    # the host share of a one-GPU box is 16 cores, whatever os.cpu_count() reports there
-    threads = min(16, os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    # every host core the process may use: os.cpu_count(), unless the machine caps the thread pools
+    # through OMP_NUM_THREADS (a one-GPU box of this pool exports 16, its share of the host)
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    threads = os.cpu_count() or 1
+    threads_note = "os.cpu_count()"
+    if cap.isdigit() and 0 < int(cap) < threads:
+        threads, threads_note = int(cap), f"OMP_NUM_THREADS={cap} set by the machine (os.cpu_count() = {os.cpu_count()})"
     torch.set_num_threads(threads)
     mode = oracle.HIER if mode_name == "hier" else oracle.TOPK
     W, b = inputs[1].cpu(), inputs[3].cpu()
@@ -161,13 +185,19 @@ def cpu_baseline(torch, mode_name, inputs, full_B, rows=0):
     while len(times) < 3 and (time.perf_counter() - t_all) < 20.0:
         times.append(run(rows))
     sec = sum(times) / len(times)
+    std = (sum((x - sec) ** 2 for x in times) / max(1, len(times) - 1)) ** 0.5
+    extrapolated = rows < full_B
     return {
         "value": round(sec * 1e3 * (full_B / rows), 1),
         "unit": "ms",
         "cores": threads,
+        "cores_from": threads_note,
         "kind": "port",
+        "extrapolated": extrapolated,
+        "std_ms": round(std * 1e3 * (full_B / rows), 1),
         "sample": f"first {rows} of {full_B} rows with the full F x D weight, {len(times)} timed fwd+bwd "
-                  f"repetitions after a warm-up, {sec * 1e3:.1f} ms each; value = that x {full_B}/{rows}",
+                  f"repetitions after a warm-up, {sec * 1e3:.1f} ms each"
+                  + (f"; value is EXTRAPOLATED to the full batch: that x {full_B}/{rows}" if extrapolated else ""),
     }
 
 
@@ -194,7 +224,7 @@ def main():
         B, K, F, D = (int(x) for x in args.shape.split(","))
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[dt_name]
     es = 2 if dtype == torch.bfloat16 else 4
-    inputs = make_inputs(torch, B, K, F, D, dtype, dist, w_std, dev)
+    inputs, generated_with = make_inputs(torch, B, K, F, D, dtype, dist, w_std, dev)
     idx, W, v, b, t = inputs
     torch.cuda.synchronize()
     abytes = algorithmic_bytes(B, K, F, D, es, es, es)
@@ -209,7 +239,8 @@ def main():
 
     torch.cuda.reset_peak_memory_stats()
     base_mem = torch.cuda.memory_allocated()
-    hier_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
+    hier_ms, hier_ev_ms, hier_std = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps,
+                                               args.warmup)
     hier_peak = torch.cuda.max_memory_allocated() - base_mem
     Wp.grad = vp.grad = bp.grad = None
     # the same step in the other memory mode of the API: with a stage budget that holds all per-pair
@@ -222,12 +253,13 @@ def main():
         flex.set_hier_stage_bytes(0 if main_staged else torch.cuda.get_device_properties(dev).total_memory // 8)
         if bool(flex.ops._stage_fits(idx, W)) != main_staged:
             torch.cuda.reset_peak_memory_stats()
-            other_ms = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps, args.warmup)
+            other_ms, _, _ = time_steps(torch, lambda: step(flex.triton_hierarchical_sae_loss), args.steps,
+                                        args.warmup)
             other_peak = torch.cuda.max_memory_allocated() - base_mem
         flex.set_hier_stage_bytes(stage_budget)
     Wp.grad = vp.grad = bp.grad = None
     torch.cuda.reset_peak_memory_stats()
-    topk_ms = time_steps(torch, lambda: step(flex.triton_topk_sae_loss), args.steps, args.warmup)
+    topk_ms, topk_ev_ms, topk_std = time_steps(torch, lambda: step(flex.triton_topk_sae_loss), args.steps, args.warmup)
     topk_peak = torch.cuda.max_memory_allocated() - base_mem
     Wp.grad = vp.grad = bp.grad = None
 
@@ -255,7 +287,7 @@ def main():
              and bool(lib.flexsae_hier_fwd_bwd_supported(ctypes.byref(sh))))
     staged = fused and flex.ops._stage_fits(idx, W)
     hier_mode = "staged" if staged else "sliced" if fused else "unfused"
-    slice_cols = D if staged else max(1, scratch // (B * K * p_size))
+    slice_cols = D if staged else flex.ops._hier_slice_cols(B, K, p_size)
     tile = 64 * (4 if D % 4 == 0 else 2 if D % 2 == 0 else 1)
     d_pad = -(-D // tile) * tile
     if fused:
@@ -334,13 +366,24 @@ def main():
     # (the training-step kernel reads bias/target instead of the residual: same order of bytes)
     sweep_launch_bytes = (B * K * D * es + B * K * (8 + es + 4) * n_slices + B * D * 4) / n_slices
     sweep_launch_ms = sweep_ms / n_slices
+    # HBM-side bytes per launch of the dominant kernel: a counter measurement (two rocprofv3 --pmc
+    # runs of this script, FETCH_SIZE and WRITE_SIZE) kept in profiles/hbm_traffic.json under the
+    # workload, the slice budget and the id of the build it was taken on.  A record of another build
+    # is not reported as this build's traffic.
     traffic = None
+    traffic_key = f"{args.workload}:{'fused' if staged else scratch >> 20}"
+    traffic_source = None
     traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    build_id = _lib.build_id()
     if os.path.exists(traffic_file) and not args.shape:
         with open(traffic_file) as fh:
-            rec = json.load(fh).get(f"{args.workload}:{'fused' if staged else scratch >> 20}")
-        if rec:
+            rec = json.load(fh).get(traffic_key)
+        if rec and rec.get("build_id") == build_id:
             traffic = rec.get(f"{sweep_name}_bytes_per_launch")
+            traffic_source = f"profiles/hbm_traffic.json[{traffic_key}], build {build_id}"
+        elif rec:
+            traffic_source = (f"none: profiles/hbm_traffic.json[{traffic_key}] was measured on build "
+                              f"{rec.get('build_id')}, this is build {build_id}")
     roofline = {
         "bound": "hbm",
         "kernel": sweep_name,
@@ -349,6 +392,7 @@ def main():
         "unit": "GB/s",
         "frac": round(gbps(sweep_launch_bytes, sweep_launch_ms) / HBM_PEAK_GBPS, 4),
         "traffic": traffic,
+        "traffic_source": traffic_source,
         "algorithmic_bytes_per_launch": int(sweep_launch_bytes),
         "avg_launch_ms": round(sweep_launch_ms, 4),
         "launches_per_step": n_slices,
@@ -362,11 +406,14 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(hier_ms, 4),
+        "ms_per_step_std": round(hier_std, 4),
+        "ms_per_step_events": round(hier_ev_ms, 4),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32 arithmetic on %s storage" % dt_name,
-        "data": "synthetic",
+        "data": "synthetic (seed 1234, %s)" % generated_with,
+        "build_id": build_id,
         "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
                                f"indices {dist}", "B": B, "K": K, "F": F, "D": D,
                    "hier_scratch_mb": scratch >> 20, "fused_training_step": bool(fused), "hier_mode": hier_mode,
@@ -388,7 +435,8 @@ def main():
             "%s x%d" % (sweep_name, n_slices): {"ms": round(sweep_ms, 4)},
             "segment reduction x%d" % n_slices: {"ms": round(reduce_ms, 4)},
         },
-        "topk": {"ms_per_step": round(topk_ms, 4), "algorithmic_bytes": abytes["topk_step"],
+        "topk": {"ms_per_step": round(topk_ms, 4), "ms_per_step_std": round(topk_std, 4),
+                 "ms_per_step_events": round(topk_ev_ms, 4), "algorithmic_bytes": abytes["topk_step"],
                  "achieved_GBps": round(gbps(abytes["topk_step"], topk_ms), 1)},
         "hier_over_topk_latency": round(hier_ms / topk_ms, 3),
         ("hier_flat_memory_mode" if main_staged else "hier_staged_mode"): None if other_ms is None else {

@@ -58,6 +58,7 @@ _shape_p = ctypes.POINTER(Shape)
 # name -> (restype, argtypes); one entry per declaration in include/flexsae_amd.h
 SIGNATURES = {
     "flexsae_abi_version": (_int, []),
+    "flexsae_build_id": (ctypes.c_char_p, []),
     "flexsae_status_string": (ctypes.c_char_p, [_int]),
     "flexsae_fwd_workspace_bytes": (_sz, [_shape_p]),
     "flexsae_hier_fwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _p, _p]),
@@ -107,6 +108,11 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} has ABI version {lib.flexsae_abi_version()}, expected {ABI_VERSION}; rebuild it")
     _lib = lib
     return lib
+
+
+def build_id() -> str:
+    """Hash of the sources and flags the loaded library was built from (flexsae_amd/build.py)."""
+    return load().flexsae_build_id().decode()
 
 
 def status_string(code: int) -> str:

@@ -24,9 +24,27 @@ HIPCC_FLAGS = [
 ]
 
 
+def source_id(extra_flags=()) -> str:
+    """Identifier of what the library is built from: a hash over the kernel sources, the header and
+    the compiler flags (not over the binary, so that rebuilding the same sources gives the same id).
+    The library reports it through flexsae_build_id(); measurements kept under profiles/ carry it."""
+    import hashlib
+
+    h = hashlib.sha256()
+    files = sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".hpp")))
+    files.append(os.path.join(os.path.dirname(HERE), "include", "flexsae_amd.h"))
+    for path in files:
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    h.update(" ".join([*HIPCC_FLAGS, *extra_flags]).encode())
+    return h.hexdigest()[:16]
+
+
 def build(verbose: bool = False, extra_flags=()) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-o", LIB_PATH, os.path.join(CSRC, "flexsae_amd.hip")]
+    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, f'-DFLEXSAE_BUILD_ID="{source_id(extra_flags)}"', "-o", LIB_PATH,
+           os.path.join(CSRC, "flexsae_amd.hip")]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)

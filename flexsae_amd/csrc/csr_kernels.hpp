@@ -197,7 +197,7 @@ __device__ __forceinline__ void block_bitonic_sort(Ptr a, uint32_t n) {
 // to kSortLdsElems pairs are sorted in LDS, longer ones in place in global memory.  With `slot`
 // given, the positions of the group's pairs are written there as well.
 constexpr uint32_t kSortLdsElems = 8192;
-__global__ __launch_bounds__(256) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
+__global__ __launch_bounds__(1024) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
                                                             uint32_t *__restrict__ map,
                                                             const uint32_t *__restrict__ long_count,
                                                             const uint32_t *__restrict__ long_list,

@@ -29,6 +29,9 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 #ifndef FLEXSAE_REDUCE_U
 #define FLEXSAE_REDUCE_U 4
 #endif
+#ifndef FLEXSAE_PIECE_U
+#define FLEXSAE_PIECE_U 4
+#endif
 #ifndef FLEXSAE_FWD_U
 #define FLEXSAE_FWD_U 8
 #endif
@@ -336,7 +339,7 @@ void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
                        n_pairs, F, pl.shift, pl.n_buckets, pl.chunk, pl.n_chunks, sc.table, sc.tmp);
     hipLaunchKernelGGL(csr_bucket_sort_kernel, dim3(pl.n_buckets), dim3(kSortThreads), 0, st, sc.tmp, sc.table,
                        pl.n_chunks, pl.shift, F, begin, map, slot, sc.long_count, sc.long_list);
-    hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(256), 0, st, begin, map, sc.long_count,
+    hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(1024), 0, st, begin, map, sc.long_count,
                        sc.long_list, slot);
     return;
   }
@@ -354,7 +357,7 @@ void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
   hipLaunchKernelGGL(csr_sort_short_kernel,
                      dim3(static_cast<unsigned>(ceil_div(F, kWavesPerBlock))), dim3(kBlock), 0, st,
                      begin, map, F, sc.long_count, sc.long_list);
-  hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(256), 0, st, begin, map, sc.long_count,
+  hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(1024), 0, st, begin, map, sc.long_count,
                      sc.long_list, static_cast<uint32_t *>(nullptr));
   if (slot)
     hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, map, n_pairs,
@@ -512,11 +515,11 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
   if (piece_cols > 0) {  // 256-byte pieces, sixteen lanes each
     const int pps = static_cast<int>(cols / piece_cols);
     const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(F * pps, kBlock / kPieceLanes));
-    hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks),
+    hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_PIECE_U>), dim3(kLongBlocks + n_short_blocks),
                        dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale,
                        F, kLongBlocks, pps, col0, sw, D);
-    // the chunk partials of hot latents are combined per 64-column tile
-    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, 1, 8>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
+    // the chunk partials of hot latents are combined per 64-column piece
+    hipLaunchKernelGGL((seg_reduce_piece_finalize_kernel<GT>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
                        sc.long_list, chunk_begin, partial, dW, dw_scale, static_cast<int>(cols / kWave), col0, sw, D);
     return;
   }
@@ -767,6 +770,11 @@ void launch_topk_slices_w(const flexsae_shape *s, const TopkBwdPlan &pl, int64_t
 extern "C" {
 
 int flexsae_abi_version(void) { return FLEXSAE_ABI_VERSION; }
+
+#ifndef FLEXSAE_BUILD_ID
+#define FLEXSAE_BUILD_ID "unknown"
+#endif
+const char *flexsae_build_id(void) { return FLEXSAE_BUILD_ID; }
 
 const char *flexsae_status_string(int status) {
   switch (status) {

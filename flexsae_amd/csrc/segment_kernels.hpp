@@ -144,16 +144,18 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
   const int group = static_cast<int>(threadIdx.x) / kPieceLanes;
   const S *__restrict__ Pp = static_cast<const S *>(P);
 
-  // acc += rows [r0, r0+n) of P at the lane's columns; n differs between the groups of a wavefront
-  auto accumulate = [&](int64_t r0, int n, int pc, float (&acc)[EV]) {
+  // acc += rows r0, r0+step, ... (n of them) of P at the lane's columns; n differs between the
+  // groups of a wavefront
+  auto accumulate = [&](int64_t r0, int n, int step, int pc, float (&acc)[EV]) {
     const S *row = Pp + r0 * slice_w + pc;
+    const int64_t stride = static_cast<int64_t>(step) * slice_w;
     for (int j = 0; __any(j < n); j += U) {
       raw_vec_t<PT, EV> raw[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         raw[u] = raw_vec_t<PT, EV>{};
         if (j + u < n)
-          raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw_vec_t<PT, EV> *>(row + static_cast<int64_t>(j + u) * slice_w));
+          raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw_vec_t<PT, EV> *>(row + (j + u) * stride));
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -166,9 +168,15 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
   };
 
   if (blockIdx.x >= n_long_blocks) {
-    const int64_t item = static_cast<int64_t>(blockIdx.x - n_long_blocks) * kGroupsPerBlock + group;
-    const int64_t f = item / pps;
-    const int t = static_cast<int>(item - f * pps);
+    // (latent, piece) of this group of lanes.  The block's first item is split with one
+    // wave-uniform division; the sixteen groups then only divide a number below pps + 16 (a 64-bit
+    // division per lane would cost more instructions than the rest of a short item)
+    const int64_t item0 = static_cast<int64_t>(blockIdx.x - n_long_blocks) * kGroupsPerBlock;
+    const int64_t f_first = item0 / pps;
+    const uint32_t rem = static_cast<uint32_t>(item0 - f_first * pps) + static_cast<uint32_t>(group);
+    const uint32_t q = rem / static_cast<uint32_t>(pps);
+    const int64_t f = f_first + q;
+    const int t = static_cast<int>(rem - q * static_cast<uint32_t>(pps));
     uint32_t s0 = 0, n = 0;
     if (f < F) {
       s0 = begin[f];
@@ -180,7 +188,7 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
     float acc[EV];
 #pragma unroll
     for (int i = 0; i < EV; ++i) acc[i] = 0.f;
-    accumulate(s0, mine ? static_cast<int>(n) : 0, pc, acc);
+    accumulate(s0, mine ? static_cast<int>(n) : 0, 1, pc, acc);
     if (scale) {  // the rows were produced for a unit upstream gradient
       const float g = scale[0];
 #pragma unroll
@@ -189,22 +197,75 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
     if (mine && d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
     return;
   }
+  // Long latents: one wavefront per (64-row chunk, piece); its four groups take every fourth row
+  // (sixteen rows in flight per wavefront) and their sums are added across the groups in a fixed
+  // order.  A hot latent's chunks are spread over many wavefronts.
   const uint32_t n_long = *long_count;
   if (n_long == 0) return;
+  constexpr int kGroups = kWave / kPieceLanes;
   const int64_t total = static_cast<int64_t>(chunk_begin[n_long]) * pps;
-  const int64_t n_groups = static_cast<int64_t>(n_long_blocks) * kGroupsPerBlock;
-  for (int64_t w = static_cast<int64_t>(blockIdx.x) * kGroupsPerBlock + group; __any(w < total); w += n_groups) {
-    const bool valid = w < total;
-    const int64_t ww = valid ? w : 0;
-    const uint32_t chunk = static_cast<uint32_t>(ww / pps);
-    const int t = static_cast<int>(ww - static_cast<int64_t>(chunk) * pps);
+  const int64_t n_waves = static_cast<int64_t>(n_long_blocks) * (blockDim.x >> 6);
+  const int g = (static_cast<int>(threadIdx.x) & (kWave - 1)) / kPieceLanes;
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total; w += n_waves) {
+    const uint32_t chunk = static_cast<uint32_t>(w / pps);
+    const int t = static_cast<int>(w - static_cast<int64_t>(chunk) * pps);
     const LongChunk c = seg_decode_chunk(begin, long_list, chunk_begin, n_long, chunk);
+    const int rows = static_cast<int>(c.s1 - c.s0);
     const int pc = t * (kPieceLanes * EV) + sub * EV;
     float acc[EV];
 #pragma unroll
     for (int i = 0; i < EV; ++i) acc[i] = 0.f;
-    accumulate(c.s0, valid ? static_cast<int>(c.s1 - c.s0) : 0, pc, acc);
-    if (valid) store_vec<float, EV>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
+    accumulate(static_cast<int64_t>(c.s0) + g, (rows - g + kGroups - 1) / kGroups, kGroups, pc, acc);
+#pragma unroll
+    for (int i = 0; i < EV; ++i) acc[i] = add_across_rows(acc[i]);
+    if (g == 0) store_vec<float, EV>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
+  }
+}
+
+// Long latents of the piece reduction, second launch: out[f, slice] = sum of the latent's chunk
+// partials in a fixed order.  One wavefront per (long latent, 64-column piece of the fp32
+// partials); its four groups take every fourth chunk and are added up as above.
+template <typename GT>
+__global__ __launch_bounds__(256) void seg_reduce_piece_finalize_kernel(
+    const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
+    const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
+    void *__restrict__ out, const float *__restrict__ scale, int pieces, int col0, int slice_w, int D) {
+  constexpr int EV = 4, U = 4, kGroups = kWave / kPieceLanes;
+  const int lane = lane_id();
+  const int sub = lane & (kPieceLanes - 1), g = lane / kPieceLanes;
+  const uint32_t n_long = *long_count;
+  const int64_t total = static_cast<int64_t>(n_long) * pieces;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total; w += n_waves) {
+    const uint32_t i = static_cast<uint32_t>(w / pieces);
+    const int t = static_cast<int>(w - static_cast<int64_t>(i) * pieces);
+    const int pc = t * (kPieceLanes * EV) + sub * EV;
+    const int d0 = col0 + pc;
+    const uint32_t c0 = chunk_begin[i], c1 = chunk_begin[i + 1];
+    const int n = (static_cast<int>(c1 - c0) - g + kGroups - 1) / kGroups;
+    const float *row = partial + (static_cast<int64_t>(c0) + g) * slice_w + pc;
+    const int64_t stride = static_cast<int64_t>(kGroups) * slice_w;
+    float acc[EV] = {0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; __any(j < n); j += U) {
+      vec_t<float, EV> raw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        raw[u] = vec_t<float, EV>{};
+        if (j + u < n) raw[u] = *reinterpret_cast<const vec_t<float, EV> *>(row + (j + u) * stride);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int k = 0; k < EV; ++k) acc[k] += raw[u][k];
+    }
+#pragma unroll
+    for (int k = 0; k < EV; ++k) acc[k] = add_across_rows(acc[k]);
+    if (scale) {
+      const float gs = scale[0];
+#pragma unroll
+      for (int k = 0; k < EV; ++k) acc[k] *= gs;
+    }
+    if (g == 0 && d0 < D) store_vec<GT, EV>(out, static_cast<int64_t>(long_list[i]) * D + d0, acc);
   }
 }
 

@@ -177,6 +177,23 @@ topk_fwd.register_fake(_fwd_fake)
 _hier_scratch_bytes = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
 
 
+# Narrowest slice the scratch budget may lead to on its own: slices below 256 columns run slower
+# (more launches, each too short to overlap its gather, arithmetic and store phases), so a budget
+# that gives fewer columns is exceeded up to this width unless `set_hier_min_slice_cols` lowers it.
+_hier_min_slice_cols = int(os.environ.get("FLEXSAE_HIER_MIN_SLICE_COLS", "256"))
+
+
+def set_hier_min_slice_cols(cols: int) -> None:
+    """Narrowest column slice of the sliced hierarchical step (default 256).  128 (16-bit weights)
+    halves the scratch of large problems at a cost of 5-10 % of the step time."""
+    global _hier_min_slice_cols
+    _hier_min_slice_cols = max(1, int(cols))
+
+
+def _hier_slice_cols(B: int, K: int, p_size: int) -> int:
+    return max(_hier_min_slice_cols, _hier_scratch_bytes // (B * K * p_size), 1)
+
+
 def set_hier_scratch_bytes(nbytes: int) -> None:
     """Upper bound on the scratch of the hierarchical backward (bytes).  0 = use the atomic
     scatter fallback, which needs no scratch but an fp32 [F,D] accumulator.  The default (256 MiB)
@@ -284,7 +301,7 @@ def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
         if _hier_scratch_bytes > 0:
             p_size = 2 if weight.dtype == torch.bfloat16 else 4
-            slice_cols = max(1, _hier_scratch_bytes // (B * K * p_size))
+            slice_cols = _hier_slice_cols(B, K, p_size)
             ws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
             workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             dW = torch.empty_like(weight)
@@ -530,7 +547,7 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
         p_size = 2 if weight.dtype == torch.bfloat16 else 4
-        slice_cols = max(1, _hier_scratch_bytes // (B * K * p_size))
+        slice_cols = _hier_slice_cols(B, K, p_size)
         ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)

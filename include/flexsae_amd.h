@@ -86,6 +86,9 @@ typedef struct {
 } flexsae_shape;
 
 int flexsae_abi_version(void);
+/* Identifier of the sources and compiler flags the library was built from (a 16-digit hash set by
+ * the build script; "unknown" for other builds): lets a stored measurement name the build it is of. */
+const char *flexsae_build_id(void);
 const char *flexsae_status_string(int status);
 
 /* Bytes of workspace the two forward entry points need for `shape`. */

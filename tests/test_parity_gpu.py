@@ -645,6 +645,78 @@ def test_opcheck_and_compile(mode):
         assert rel_err(W.grad.cpu(), want.cpu().numpy()) < 1e-5
 
 
+def test_opcheck_of_every_op_with_all_checks():
+    """torch.library.opcheck with its full default set of checks (schema, autograd registration,
+    fake tensors, AOT dispatch with dynamic shapes) on every op of the package."""
+    idx, W, v, b, t = _to_dev(make_inputs(16, 8, 40, 256, seed=6))
+    ops = torch.ops.flexsae_amd
+    g = torch.tensor(0.7, device=DEV)
+
+    def leaves():
+        return [x.clone().requires_grad_() for x in (W, v, b)]
+
+    for op in (ops.hier_fwd, ops.topk_fwd, ops.hier_train_sliced):
+        Wl, vl, bl = leaves()
+        torch.library.opcheck(op, (idx, Wl, vl, bl, t))
+    _, vl, bl = leaves()
+    torch.library.opcheck(ops.hier_train_sliced, (idx, W, vl, bl, t, False))  # a frozen decoder
+    # hier_train's fourth output is its workspace (scratch whose unwritten bytes differ from run to
+    # run), so opcheck's eager-vs-traced comparison of ALL outputs cannot hold for it: the other
+    # three checks run as they are, and the AOT-dispatch check with dynamic shapes is run on the
+    # three outputs that are defined, gradients included
+    Wl, vl, bl = leaves()
+    torch.library.opcheck(ops.hier_train, (idx, Wl, vl, bl, t),
+                          test_utils=("test_schema", "test_autograd_registration", "test_faketensor"))
+
+    def defined_outputs(i, w, vv, bb, tt):
+        loss, dvals, dbias, _ = ops.hier_train(i, w, vv, bb, tt)
+        return loss, dvals, dbias
+
+    eager_l = leaves()
+    eager = defined_outputs(idx, *eager_l, t)
+    eager[0].backward()
+    traced_l = leaves()
+    torch._dynamo.reset()
+    traced = torch.compile(defined_outputs, backend="aot_eager", dynamic=True, fullgraph=True)(idx, *traced_l, t)
+    traced[0].backward()
+    for a, c in zip(eager, traced):
+        assert torch.equal(a, c)
+    for a, c in zip(eager_l, traced_l):
+        assert torch.equal(a.grad, c.grad)
+    _, resid_h = ops.hier_fwd(idx, W, v, b, t)
+    _, resid_t = ops.topk_fwd(idx, W, v, b, t)
+    torch.library.opcheck(ops.hier_bwd, (g, idx, W, v, resid_h))
+    torch.library.opcheck(ops.topk_bwd, (g, idx, W, v, resid_t))
+    stage = ops.hier_train(idx, W, v, b, t)[3]
+    torch.library.opcheck(ops.hier_finish, (g, idx, W, v, stage))
+    torch.library.opcheck(ops.scale_by, (W, g))
+    torch.library.opcheck(ops.scale_, (W.clone(), g))
+
+
+@pytest.mark.parametrize("mode", ["hier", "topk"])
+def test_compile_with_the_default_backend(mode):
+    """torch.compile(fullgraph=True) with the default backend (inductor) around the fused loss, as
+    a caller compiling the training step would (reference example.py:15 compiles its competitor):
+    same loss and gradients as eager."""
+    args = make_inputs(32, 16, 96, 512, seed=9)
+    idx, W, v, b, t = _to_dev(args)
+    leaves_e = [x.clone().requires_grad_() for x in (W, v, b)]
+    leaves_c = [x.clone().requires_grad_() for x in (W, v, b)]
+
+    def fn(i, w, vv, bb, tt):
+        return FUSED[mode](i, w, vv * 1.5, bb, tt) * 2.0 + 1.0
+
+    eager = fn(idx, *leaves_e, t)
+    eager.backward()
+    torch._dynamo.reset()
+    compiled = torch.compile(fn, fullgraph=True)(idx, *leaves_c, t)
+    compiled.backward()
+    torch.cuda.synchronize()
+    assert abs(compiled.item() - eager.item()) <= 1e-6 * abs(eager.item())
+    for ge, gc in zip(leaves_e, leaves_c):
+        assert gc.grad is not None and rel_err(gc.grad.cpu(), ge.grad.cpu().numpy()) < 1e-5
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("order", ["topk_first", "hier_first"])
 @pytest.mark.parametrize("fused", ["sliced", "staged", "unfused"])
