@@ -515,9 +515,12 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
   if (piece_cols > 0) {  // 256-byte pieces, sixteen lanes each
     const int pps = static_cast<int>(cols / piece_cols);
     const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(F * pps, kBlock / kPieceLanes));
+    int pps_shift = -1;  // log2(pps) when pps is a power of two
+    for (int sh = 0; sh < 16; ++sh)
+      if (pps == (1 << sh)) pps_shift = sh;
     hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_PIECE_U>), dim3(kLongBlocks + n_short_blocks),
                        dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale,
-                       F, kLongBlocks, pps, col0, sw, D);
+                       F, kLongBlocks, pps, pps_shift, col0, sw, D);
     // the chunk partials of hot latents are combined per 64-column piece
     hipLaunchKernelGGL((seg_reduce_piece_finalize_kernel<GT>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
                        sc.long_list, chunk_begin, partial, dW, dw_scale, static_cast<int>(cols / kWave), col0, sw, D);
@@ -569,20 +572,35 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   // columns that are worked on: whole reduction tiles, or, with the piece reduction, whole training
   // tiles (tiles that lie entirely beyond column D are left out, and so are their shares below)
   const int64_t d_used = hier_cols_used(s, pl, train != nullptr, piece != 0);
+  // The sweep kernel's tile (64 * sweep_vec columns per wavefront): narrower than the reduction's
+  // when a slice would otherwise hold too few wavefronts to cover the memory latency (small B).
+  // (not below the tile width the per-tile dvals shares of the workspace are laid out for)
+  int sweep_vec = VEC;
+  const int min_sweep_vec = static_cast<int>((pl.tile < train_tile_cols(s) ? pl.tile : train_tile_cols(s)) / kWave);
+  while (sweep_vec > 1 && sweep_vec > min_sweep_vec && s->B * (slice_w / (kWave * sweep_vec)) < 6144) sweep_vec >>= 1;
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (d_used - col0) < slice_w ? (d_used - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
-    const int64_t sweep_items = s->B * tps;
     if (train && do_sweep) {
       launch_train_kernel_k<WT, PT>(s, *train, indices, weight, vals, coef, slot, P, dv_part, s_final, d_pad,
                                     reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
                                     static_cast<int>(col0), sw, st);
-    } else if (do_sweep)
-      hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, VEC, FLEXSAE_SWEEP_U>),
-                         dim3(static_cast<unsigned>(ceil_div(sweep_items, kWavesPerBlock))), dim3(kBlock),
-                         0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, dv_part,
-                         s_final, d_pad, status_flag, sweep_items, s->B, static_cast<int>(col0), sw, K, s->F,
-                         D);
+    } else if (do_sweep) {
+#define FLEXSAE_SWEEP(SV)                                                                                      \
+  hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, SV, FLEXSAE_SWEEP_U>),                                         \
+                     dim3(static_cast<unsigned>(ceil_div(s->B * (cols / (kWave * SV)), kWavesPerBlock))),      \
+                     dim3(kBlock), 0, st, indices, weight, vals, s->vals_dtype, resid, grad_out, coef, slot, P, \
+                     dv_part, s_final, d_pad, status_flag, s->B * (cols / (kWave * SV)), s->B,                 \
+                     static_cast<int>(col0), sw, K, s->F, D)
+      if (sweep_vec == VEC) {
+        FLEXSAE_SWEEP(VEC);
+      } else if (sweep_vec == (VEC >= 2 ? VEC / 2 : 1)) {
+        FLEXSAE_SWEEP((VEC >= 2 ? VEC / 2 : 1));
+      } else {
+        FLEXSAE_SWEEP(1);
+      }
+#undef FLEXSAE_SWEEP
+    }
     if (!do_reduce) continue;
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
                                    static_cast<int>(col0), sw, D, st, piece, cols);
@@ -592,7 +610,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   if (flags & FLEXSAE_BWD_SKIP_EPILOGUE) return;
   // dvals = its per-tile shares added in tile order
   hipLaunchKernelGGL(hier_dvals_finalize_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, dv_part,
-                     static_cast<int>(d_used / (train ? train_tile_cols(s) : pl.tile)), s->B * s->K, dvals);
+                     static_cast<int>(d_used / (train ? train_tile_cols(s) : kWave * sweep_vec)), s->B * s->K, dvals);
   // dbias = column sums of s_final over the rows, in a fixed order
   hipLaunchKernelGGL(colsum_partial_kernel,
                      dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),

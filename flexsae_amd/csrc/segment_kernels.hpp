@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
     const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
     const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
     const void *__restrict__ P, float *__restrict__ partial, void *__restrict__ out,
-    const float *__restrict__ scale, int64_t F, unsigned n_long_blocks, int pps, int col0,
+    const float *__restrict__ scale, int64_t F, unsigned n_long_blocks, int pps, int pps_shift, int col0,
     int slice_w, int D) {
   using S = typename Traits<PT>::store_t;
   constexpr int EV = 16 / static_cast<int>(sizeof(S));  // columns per lane
@@ -172,11 +172,19 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
     // wave-uniform division; the sixteen groups then only divide a number below pps + 16 (a 64-bit
     // division per lane would cost more instructions than the rest of a short item)
     const int64_t item0 = static_cast<int64_t>(blockIdx.x - n_long_blocks) * kGroupsPerBlock;
-    const int64_t f_first = item0 / pps;
-    const uint32_t rem = static_cast<uint32_t>(item0 - f_first * pps) + static_cast<uint32_t>(group);
-    const uint32_t q = rem / static_cast<uint32_t>(pps);
-    const int64_t f = f_first + q;
-    const int t = static_cast<int>(rem - q * static_cast<uint32_t>(pps));
+    int64_t f;
+    int t;
+    if (pps_shift >= 0) {  // pps is a power of two (the usual slice widths): shifts only
+      const int64_t item = item0 + group;
+      f = item >> pps_shift;
+      t = static_cast<int>(item & ((1 << pps_shift) - 1));
+    } else {
+      const int64_t f_first = item0 / pps;
+      const uint32_t rem = static_cast<uint32_t>(item0 - f_first * pps) + static_cast<uint32_t>(group);
+      const uint32_t q = rem / static_cast<uint32_t>(pps);
+      f = f_first + q;
+      t = static_cast<int>(rem - q * static_cast<uint32_t>(pps));
+    }
     uint32_t s0 = 0, n = 0;
     if (f < F) {
       s0 = begin[f];
