@@ -277,7 +277,7 @@ def main():
     dbias = torch.empty(D, dtype=torch.float32, device=dev)
     dW = torch.empty(F, D, dtype=dtype, device=dev)
     p_size = 2 if dtype == torch.bfloat16 else 4
-    scratch = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
+    scratch = flex.ops._hier_scratch_budget(K)  # FLEXSAE_HIER_SCRATCH_MB, else the package's default rule
     # same decision as the API: the fused training step runs when the stage budget holds every
     # per-pair contribution at once (one slice as wide as D); otherwise forward + sliced backward
     # (staged); failing that, the same kernel slice by slice with an immediate reduction (sliced);

@@ -448,8 +448,8 @@ struct TrainArgs {
   const void *target;
 };
 
-// largest K the training-step kernel holds in registers, per weight dtype
-inline bool train_supported(const flexsae_shape *s) { return s->D % 4 == 0 && s->K <= 128; }
+// largest K the training-step kernel holds in registers
+inline bool train_supported(const flexsae_shape *s) { return s->D % 4 == 0 && s->K <= 256; }
 
 template <typename WT, typename PT, int KMAX, int VEC = 2>
 void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
@@ -486,9 +486,16 @@ void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const in
   } else if (s->K <= 64) {
     FLEXSAE_TRAIN(64);
   } else if constexpr (sizeof(typename Traits<WT>::store_t) == 2) {
-    FLEXSAE_TRAIN(128);
-  } else {  // fp32 rows of 65..128 steps: one column per lane
+    if (s->K <= 128) {
+      FLEXSAE_TRAIN(128);
+    } else {  // 129..256 steps: one wavefront per SIMD, part of the row pieces in accumulation registers
+      FLEXSAE_TRAIN(256);
+    }
+  } else if (s->K <= 128) {  // fp32 rows of 65..128 steps: one column per lane
     launch_train_kernel<WT, PT, 128, 1>(s, ta, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,
+                                        loss_partial, status_flag, cols, col0, slice_w, st);
+  } else {
+    launch_train_kernel<WT, PT, 256, 1>(s, ta, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,
                                         loss_partial, status_flag, cols, col0, slice_w, st);
   }
 #undef FLEXSAE_TRAIN
