@@ -518,16 +518,27 @@ size_t hier_bwd_bytes(const HierBwdPlan &p, int64_t slice_w) {
 template <typename PT, typename GT, int VEC>
 void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc, const uint32_t *chunk_begin,
                        const void *P, float *partial, void *dW, const float *dw_scale, int64_t F, int tps,
-                       int col0, int sw, int D, hipStream_t st, int piece_cols = 0, int64_t cols = 0) {
+                       int col0, int sw, int D, hipStream_t st, int piece_cols = 0, int64_t cols = 0, int64_t n_pairs = 0) {
   if (piece_cols > 0) {  // 256-byte pieces, sixteen lanes each
     const int pps = static_cast<int>(cols / piece_cols);
-    const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(F * pps, kBlock / kPieceLanes));
     int pps_shift = -1;  // log2(pps) when pps is a power of two
     for (int sh = 0; sh < 16; ++sh)
       if (pps == (1 << sh)) pps_shift = sh;
-    hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_PIECE_U>), dim3(kLongBlocks + n_short_blocks),
-                       dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale,
-                       F, kLongBlocks, pps, pps_shift, col0, sw, D);
+    // latents per group of lanes: several where latents have few rows on average
+    const int per_group = n_pairs <= 2 * F ? 4 : n_pairs <= 4 * F ? 2 : 1;
+#define FLEXSAE_PIECE_REDUCE(G)                                                                                    \
+  hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_PIECE_U, G>),                                        \
+                     dim3(kLongBlocks + static_cast<unsigned>(ceil_div(ceil_div(F, G) * pps, kBlock / kPieceLanes))), \
+                     dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, \
+                     F, kLongBlocks, pps, pps_shift, col0, sw, D)
+    if (per_group == 4) {
+      FLEXSAE_PIECE_REDUCE(4);
+    } else if (per_group == 2) {
+      FLEXSAE_PIECE_REDUCE(2);
+    } else {
+      FLEXSAE_PIECE_REDUCE(1);
+    }
+#undef FLEXSAE_PIECE_REDUCE
     // the chunk partials of hot latents are combined per 64-column piece
     hipLaunchKernelGGL((seg_reduce_piece_finalize_kernel<GT>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
                        sc.long_list, chunk_begin, partial, dW, dw_scale, static_cast<int>(cols / kWave), col0, sw, D);
@@ -610,7 +621,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     }
     if (!do_reduce) continue;
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
-                                   static_cast<int>(col0), sw, D, st, piece, cols);
+                                   static_cast<int>(col0), sw, D, st, piece, cols, s->B * s->K);
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only

@@ -126,11 +126,12 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
 // keeps the contributions of one slice in the memory-side cache between the launch that writes them
 // and this one.  The four latents (or pieces) of a wavefront have different row counts: the loop
 // runs to the longest, loads beyond a group's own count are masked off.  Work order: pieces of a
-// latent adjacent, latents ascending, so the launch still reads P front to back.
+// latent adjacent, latents ascending, so the launch still reads P front to back.  G > 1: a group
+// serves G consecutive latents (chosen by the caller where latents have few rows on average).
 constexpr int kPieceLanes = 16;
 constexpr int kPieceBytes = kPieceLanes * 16;
 
-template <typename PT, typename GT, int U>
+template <typename PT, typename GT, int U, int G>
 __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
     const uint32_t *__restrict__ begin, const uint32_t *__restrict__ long_count,
     const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
@@ -168,41 +169,114 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
   };
 
   if (blockIdx.x >= n_long_blocks) {
-    // (latent, piece) of this group of lanes.  The block's first item is split with one
-    // wave-uniform division; the sixteen groups then only divide a number below pps + 16 (a 64-bit
-    // division per lane would cost more instructions than the rest of a short item)
+    // (latent block, piece) of this group of lanes; a latent block is G consecutive latents.  The
+    // block's first item is split with one wave-uniform division; the sixteen groups then only
+    // divide a number below pps + 16 (a 64-bit division per lane would cost more instructions than
+    // the rest of a short item)
     const int64_t item0 = static_cast<int64_t>(blockIdx.x - n_long_blocks) * kGroupsPerBlock;
-    int64_t f;
+    int64_t fb;
     int t;
     if (pps_shift >= 0) {  // pps is a power of two (the usual slice widths): shifts only
       const int64_t item = item0 + group;
-      f = item >> pps_shift;
+      fb = item >> pps_shift;
       t = static_cast<int>(item & ((1 << pps_shift) - 1));
     } else {
       const int64_t f_first = item0 / pps;
       const uint32_t rem = static_cast<uint32_t>(item0 - f_first * pps) + static_cast<uint32_t>(group);
       const uint32_t q = rem / static_cast<uint32_t>(pps);
-      f = f_first + q;
+      fb = f_first + q;
       t = static_cast<int>(rem - q * static_cast<uint32_t>(pps));
     }
-    uint32_t s0 = 0, n = 0;
-    if (f < F) {
-      s0 = begin[f];
-      n = begin[f + 1] - s0;
-    }
-    const bool mine = f < F && n <= static_cast<uint32_t>(kSegChunk);  // longer ones: chunked below
     const int pc = t * (kPieceLanes * EV) + sub * EV;
     const int d0 = col0 + pc;
+    const float g = scale ? scale[0] : 1.0f;  // the rows were produced for a unit upstream gradient
     float acc[EV];
 #pragma unroll
     for (int i = 0; i < EV; ++i) acc[i] = 0.f;
-    accumulate(s0, mine ? static_cast<int>(n) : 0, 1, pc, acc);
-    if (scale) {  // the rows were produced for a unit upstream gradient
-      const float g = scale[0];
+    if constexpr (G == 1) {
+      const int64_t f = fb;
+      uint32_t s0 = 0, n = 0;
+      if (f < F) {
+        s0 = begin[f];
+        n = begin[f + 1] - s0;
+      }
+      const bool mine = f < F && n <= static_cast<uint32_t>(kSegChunk);  // longer ones: chunked below
+      accumulate(s0, mine ? static_cast<int>(n) : 0, 1, pc, acc);
+      if (scale) {
 #pragma unroll
-      for (int i = 0; i < EV; ++i) acc[i] *= g;
+        for (int i = 0; i < EV; ++i) acc[i] *= g;
+      }
+      if (mine && d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
+    } else {
+      // Few rows per latent: a launch of one latent per group is a train of short-lived wavefronts,
+      // each waiting for two dependent round trips (begin[], then the rows).  Here a group serves G
+      // consecutive latents: their rows are adjacent in P (apart from those of a long latent in
+      // between), so they are fetched U at a time regardless of where one latent ends and the next
+      // begins, and a latent's sum is stored when its last row has been added.  The order of the
+      // additions of a latent is the same as with G = 1.
+      const int64_t f0 = fb * G;
+      uint32_t bv = 0;  // lane j of the group holds begin[f0 + j], j <= G
+      if (f0 < F && sub <= G) bv = begin[f0 + sub < F ? f0 + sub : F];
+      uint32_t c[G + 1], off[G];  // row i of the group's list, c[j] <= i < c[j+1], is row i + off[j] of P
+      bool own[G];
+      c[0] = 0;
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const uint32_t b0 = static_cast<uint32_t>(__shfl(static_cast<int>(bv), j, kPieceLanes));
+        const uint32_t b1 = static_cast<uint32_t>(__shfl(static_cast<int>(bv), j + 1, kPieceLanes));
+        const uint32_t n = b1 - b0;
+        own[j] = f0 + j < F && n <= static_cast<uint32_t>(kSegChunk);
+        c[j + 1] = c[j] + (own[j] ? n : 0u);
+        off[j] = b0 - c[j];
+      }
+      float zero[EV];
+#pragma unroll
+      for (int i = 0; i < EV; ++i) zero[i] = 0.f;
+#pragma unroll
+      for (int j = 0; j < G; ++j)  // latents without rows
+        if (own[j] && c[j + 1] == c[j] && d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, (f0 + j) * D + d0, zero);
+      const uint32_t total = c[G];
+      for (uint32_t i0 = 0; __any(i0 < total); i0 += U) {
+        raw_vec_t<PT, EV> raw[U];
+        int which[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t i = i0 + u;
+          raw[u] = raw_vec_t<PT, EV>{};
+          which[u] = 0;
+          uint32_t o = off[0];
+#pragma unroll
+          for (int j = 1; j < G; ++j)
+            if (i >= c[j]) {
+              which[u] = j;
+              o = off[j];
+            }
+          if (i < total)
+            raw[u] = __builtin_nontemporal_load(reinterpret_cast<const raw_vec_t<PT, EV> *>(
+                Pp + static_cast<int64_t>(i + o) * slice_w + pc));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t i = i0 + u;
+          float x[EV];
+          unpack_raw<PT, EV>(raw[u], x);
+#pragma unroll
+          for (int k = 0; k < EV; ++k) acc[k] += x[k];  // masked-off loads left zeros
+          bool last = false;  // the last row of its latent
+#pragma unroll
+          for (int j = 1; j <= G; ++j) last |= i + 1 == c[j];
+          if (i < total && last) {
+            if (scale) {
+#pragma unroll
+              for (int k = 0; k < EV; ++k) acc[k] *= g;
+            }
+            if (d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, (f0 + which[u]) * D + d0, acc);
+#pragma unroll
+            for (int k = 0; k < EV; ++k) acc[k] = 0.f;
+          }
+        }
+      }
     }
-    if (mine && d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
     return;
   }
   // Long latents: one wavefront per (64-row chunk, piece); its four groups take every fourth row

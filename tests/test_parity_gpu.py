@@ -119,11 +119,12 @@ def test_reference_matrix_without_fused_training(B, K, F, D, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
 @pytest.mark.parametrize("shape", [(48, 32, 200, 768), (7, 5, 300, 260), (33, 128, 64, 2304), (16, 64, 9, 132),
                                    (5, 100, 40, 512), (64, 16, 1000, 4), (9, 256, 700, 320), (6, 130, 50, 192),
-                                   (12, 200, 3000, 72)])
+                                   (12, 200, 3000, 72), (40, 16, 200, 512), (50, 8, 333, 640)])
 def test_training_step_entry_point(shape, dtype):
     """flexsae_hier_fwd_bwd through the C-ABI: loss and unit-gradient gradients in one pass, for
     K that are not powers of two (up to 256, where a wavefront keeps part of the row pieces in
-    accumulation registers), D that are not whole tiles, hot latents (F tiny)."""
+    accumulation registers), D that are not whole tiles, hot latents (F tiny), and between one and
+    four pairs per latent on average (the reduction then serves two or four latents per group of lanes)."""
     B, K, F, D = shape
     _announce("train abi", shape, dtype)
     args = make_inputs(B, K, F, D, dtype=dtype, seed=41)
