@@ -258,6 +258,17 @@ def main():
             other_peak = torch.cuda.max_memory_allocated() - base_mem
         flex.set_hier_stage_bytes(stage_budget)
     Wp.grad = vp.grad = bp.grad = None
+    # the training step with the plain-SGD update of the decoder weight fused into the reduction
+    # (no dense dW, untouched rows neither read nor written); a step size of zero keeps the weights
+    # as they are while moving the same bytes
+    sgd_ms = sgd_peak = None
+    if not args.no_other_mode and flex.ops._train_supported(W, K) and D % (4 if dtype == torch.float32 else 8) == 0:
+        zero_step = torch.zeros((), dtype=torch.float32, device=dev)
+        torch.cuda.reset_peak_memory_stats()
+        with torch.no_grad():
+            sgd_ms, _, _ = time_steps(torch, lambda: flex.ops.hier_sgd_step(idx, W, v, b, t, zero_step),
+                                      args.steps, args.warmup)
+        sgd_peak = torch.cuda.max_memory_allocated() - base_mem
     torch.cuda.reset_peak_memory_stats()
     topk_ms, topk_ev_ms, topk_std = time_steps(torch, lambda: step(flex.triton_topk_sae_loss), args.steps, args.warmup)
     topk_peak = torch.cuda.max_memory_allocated() - base_mem
@@ -442,6 +453,10 @@ def main():
         ("hier_flat_memory_mode" if main_staged else "hier_staged_mode"): None if other_ms is None else {
             "ms_per_step": round(other_ms, 4), "over_topk_latency": round(other_ms / topk_ms, 3),
             "peak_mem_gib": round(other_peak / 2 ** 30, 3)},
+        "hier_sgd_step": None if sgd_ms is None else {
+            "ms_per_step": round(sgd_ms, 4), "over_topk_latency": round(sgd_ms / topk_ms, 3),
+            "peak_mem_gib": round(sgd_peak / 2 ** 30, 3),
+            "what": "flexsae_hier_sgd_step: loss, dvals, dbias and the in-place SGD update of W; no dense dW"},
         "peak_mem_gib": {"hier": round(hier_peak / 2 ** 30, 3), "topk": round(topk_peak / 2 ** 30, 3),
                          "inputs": round(base_mem / 2 ** 30, 3)},
     }

@@ -69,6 +69,7 @@ SIGNATURES = {
     "flexsae_hier_fwd_bwd_supported": (_int, [_shape_p]),
     "flexsae_hier_fwd_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_hier_fwd_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p, _p]),
+    "flexsae_hier_sgd_step": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _int, _p, _p]),
     "flexsae_scale": (_int, [_p, _p, _int, _i64, _p, _p]),
     "flexsae_hier_bwd_atomic": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p]),
     "flexsae_csr_workspace_bytes": (_sz, [_i64, _i64, _i64]),

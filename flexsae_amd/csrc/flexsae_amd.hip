@@ -47,6 +47,7 @@ namespace {
 constexpr int kBlock = 256;              // threads per block of the wave-per-item kernels
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr size_t kAlign = 256;
+constexpr int kBwdSgdUpdate = 1 << 20;  // internal flag of the slice loop: dW is the weight matrix, updated in place
 constexpr unsigned kLongBlocks = 1024;    // leading blocks of a reduction launch that serve hot latents
 
 inline bool valid_dtype(int d) { return d == FLEXSAE_F32 || d == FLEXSAE_BF16 || d == FLEXSAE_F16; }
@@ -518,7 +519,8 @@ size_t hier_bwd_bytes(const HierBwdPlan &p, int64_t slice_w) {
 template <typename PT, typename GT, int VEC>
 void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc, const uint32_t *chunk_begin,
                        const void *P, float *partial, void *dW, const float *dw_scale, int64_t F, int tps,
-                       int col0, int sw, int D, hipStream_t st, int piece_cols = 0, int64_t cols = 0, int64_t n_pairs = 0) {
+                       int col0, int sw, int D, hipStream_t st, int piece_cols = 0, int64_t cols = 0, int64_t n_pairs = 0,
+                       int update = 0) {
   if (piece_cols > 0) {  // 256-byte pieces, sixteen lanes each
     const int pps = static_cast<int>(cols / piece_cols);
     int pps_shift = -1;  // log2(pps) when pps is a power of two
@@ -530,7 +532,7 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
   hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_PIECE_U, G>),                                        \
                      dim3(kLongBlocks + static_cast<unsigned>(ceil_div(ceil_div(F, G) * pps, kBlock / kPieceLanes))), \
                      dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, \
-                     F, kLongBlocks, pps, pps_shift, col0, sw, D)
+                     F, kLongBlocks, pps, pps_shift, col0, sw, D, update)
     if (per_group == 4) {
       FLEXSAE_PIECE_REDUCE(4);
     } else if (per_group == 2) {
@@ -541,7 +543,8 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
 #undef FLEXSAE_PIECE_REDUCE
     // the chunk partials of hot latents are combined per 64-column piece
     hipLaunchKernelGGL((seg_reduce_piece_finalize_kernel<GT>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
-                       sc.long_list, chunk_begin, partial, dW, dw_scale, static_cast<int>(cols / kWave), col0, sw, D);
+                       sc.long_list, chunk_begin, partial, dW, dw_scale, static_cast<int>(cols / kWave), col0, sw, D,
+                       update);
     return;
   }
   constexpr bool kCanNarrow = sizeof(typename Traits<PT>::store_t) == 4 && VEC == 4;
@@ -572,7 +575,9 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                         hipStream_t st, const TrainArgs *train = nullptr, int piece = 0) {
   const bool do_sweep = !(flags & FLEXSAE_BWD_REDUCE_ONLY);
   const bool do_reduce = !(flags & FLEXSAE_BWD_SWEEP_ONLY);
-  const float *dw_scale = (flags & FLEXSAE_BWD_SCALE_BY_GRAD_OUT) ? grad_out : nullptr;
+  // in-place weight update: `grad_out` is the step size and dW the weight matrix (piece reduction only)
+  const int update = (flags & kBwdSgdUpdate) ? 1 : 0;
+  const float *dw_scale = (flags & (FLEXSAE_BWD_SCALE_BY_GRAD_OUT | kBwdSgdUpdate)) ? grad_out : nullptr;
   const uint32_t *begin = reinterpret_cast<const uint32_t *>(ws + pl.off_begin);
   const uint32_t *slot = reinterpret_cast<const uint32_t *>(ws + pl.off_slot);
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
@@ -621,7 +626,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     }
     if (!do_reduce) continue;
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
-                                   static_cast<int>(col0), sw, D, st, piece, cols, s->B * s->K);
+                                   static_cast<int>(col0), sw, D, st, piece, cols, s->B * s->K, update);
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
@@ -1022,12 +1027,24 @@ int flexsae_hier_fwd_bwd_supported(const flexsae_shape *s) {
   return check_shape(s) == FLEXSAE_OK && train_supported(s) ? 1 : 0;
 }
 
-int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const void *weight,
-                         const void *vals, const void *bias, const void *target, float *loss,
-                         void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
-                         size_t workspace_bytes, int flags, int *status_flag, void *stream) {
+}  // extern "C"
+
+namespace {
+
+// flexsae_hier_fwd_bwd, or with `sgd_step` (a device scalar) flexsae_hier_sgd_step: dW is then the
+// weight matrix itself and every touched row has step * (its unit-gradient row) subtracted.
+int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void *weight,
+                      const void *vals, const void *bias, const void *target, float *loss,
+                      void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
+                      size_t workspace_bytes, int flags, int *status_flag, void *stream,
+                      const float *sgd_step) {
   int rc = check_shape(s);
   if (rc != FLEXSAE_OK) return rc;
+  if (sgd_step) {
+    if (flags & (FLEXSAE_BWD_NO_DW | FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE))
+      return FLEXSAE_ERR_INVALID_ARGUMENT;
+    if (!aligned(sgd_step, 4)) return FLEXSAE_ERR_ALIGNMENT;
+  }
   const bool no_dw = (flags & FLEXSAE_BWD_NO_DW) != 0;
   const bool defer_reduce = (flags & FLEXSAE_BWD_SWEEP_ONLY) != 0 && !no_dw;
   if (!indices || !weight || !vals || !bias || !target || !loss || !dvals || !dbias ||
@@ -1044,6 +1061,7 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   // slices are whole training tiles when the reduction can work on 256-byte pieces, else whole
   // reduction tiles
   const bool piece = piece_reduce_ok(s, pl, (defer_reduce || no_dw) ? nullptr : dW, dW_dtype);
+  if (sgd_step && !piece) return FLEXSAE_ERR_UNSUPPORTED;  // only the piece reduction updates in place
   const int64_t granule = piece ? train_tile_cols(s) : pl.tile;
   if (!workspace || !aligned(workspace, kAlign) || workspace_bytes < hier_bwd_bytes(pl, granule))
     return FLEXSAE_ERR_WORKSPACE;
@@ -1066,10 +1084,10 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
   const float coef = static_cast<float>(2.0 / count);
   const TrainArgs ta = {bias, target};
   // without dW the reductions are left out like in the deferred case (dW_dtype only selects a template then)
-  launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, nullptr, coef, dW,
+  launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, sgd_step, coef, dW,
                           no_dw ? s->weight_dtype : dW_dtype, dvals, dbias, ws,
                           (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE)) |
-                              (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0),
+                              (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0) | (sgd_step ? kBwdSgdUpdate : 0),
                           status_flag, st, &ta, piece ? static_cast<int>(piece_cols(pl)) : 0);
   rc = launch_status();
   if (rc != FLEXSAE_OK || (flags & FLEXSAE_BWD_SKIP_EPILOGUE)) return rc;
@@ -1078,6 +1096,28 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
                      s->B * (hier_cols_used(s, pl, true, piece) / train_tile_cols(s)), 1.0 / count,
                      loss);
   return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const void *weight,
+                         const void *vals, const void *bias, const void *target, float *loss,
+                         void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
+                         size_t workspace_bytes, int flags, int *status_flag, void *stream) {
+  return hier_fwd_bwd_impl(s, indices, weight, vals, bias, target, loss, dW, dW_dtype, dvals, dbias, workspace,
+                           workspace_bytes, flags & ~kBwdSgdUpdate, status_flag, stream, nullptr);
+}
+
+int flexsae_hier_sgd_step(const flexsae_shape *s, const int64_t *indices, void *weight, const void *vals,
+                          const void *bias, const void *target, const float *step, float *loss,
+                          float *dvals, float *dbias, void *workspace, size_t workspace_bytes, int flags,
+                          int *status_flag, void *stream) {
+  if (!step || !s) return FLEXSAE_ERR_INVALID_ARGUMENT;
+  return hier_fwd_bwd_impl(s, indices, weight, vals, bias, target, loss, weight, s->weight_dtype, dvals, dbias,
+                           workspace, workspace_bytes, flags & FLEXSAE_BWD_REUSE_PAIR_LIST, status_flag, stream,
+                           step);
 }
 
 int flexsae_scale(void *dst, const void *src, int dtype, int64_t n, const float *scale, void *stream) {

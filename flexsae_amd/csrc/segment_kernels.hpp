@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
     const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
     const void *__restrict__ P, float *__restrict__ partial, void *__restrict__ out,
     const float *__restrict__ scale, int64_t F, unsigned n_long_blocks, int pps, int pps_shift, int col0,
-    int slice_w, int D) {
+    int slice_w, int D, int update) {
   using S = typename Traits<PT>::store_t;
   constexpr int EV = 16 / static_cast<int>(sizeof(S));  // columns per lane
   constexpr int kGroupsPerBlock = 256 / kPieceLanes;
@@ -166,6 +166,20 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
         for (int i = 0; i < EV; ++i) acc[i] += x[i];  // masked-off loads left zeros
       }
     }
+  };
+
+  // A latent's finished sum goes to out[f, d0..]; in update mode it is subtracted from what is there
+  // (out is then the weight matrix, the sum arrives scaled by the step size, and latents without
+  // rows are left alone).
+  auto emit = [&](int64_t f, int d0, float (&acc)[EV]) {
+    if (d0 >= D) return;
+    if (update) {
+      float w[EV];
+      load_vec<GT, EV>(out, f * D + d0, w);
+#pragma unroll
+      for (int i = 0; i < EV; ++i) acc[i] = w[i] - acc[i];
+    }
+    store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
   };
 
   if (blockIdx.x >= n_long_blocks) {
@@ -206,7 +220,7 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
 #pragma unroll
         for (int i = 0; i < EV; ++i) acc[i] *= g;
       }
-      if (mine && d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, f * D + d0, acc);
+      if (mine && !(update && n == 0)) emit(f, d0, acc);
     } else {
       // Few rows per latent: a launch of one latent per group is a train of short-lived wavefronts,
       // each waiting for two dependent round trips (begin[], then the rows).  Here a group serves G
@@ -234,7 +248,8 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
       for (int i = 0; i < EV; ++i) zero[i] = 0.f;
 #pragma unroll
       for (int j = 0; j < G; ++j)  // latents without rows
-        if (own[j] && c[j + 1] == c[j] && d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, (f0 + j) * D + d0, zero);
+        if (own[j] && c[j + 1] == c[j] && d0 < D && !update)
+          store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, (f0 + j) * D + d0, zero);
       const uint32_t total = c[G];
       for (uint32_t i0 = 0; __any(i0 < total); i0 += U) {
         raw_vec_t<PT, EV> raw[U];
@@ -270,7 +285,7 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
 #pragma unroll
               for (int k = 0; k < EV; ++k) acc[k] *= g;
             }
-            if (d0 < D) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, (f0 + which[u]) * D + d0, acc);
+            emit(f0 + which[u], d0, acc);
 #pragma unroll
             for (int k = 0; k < EV; ++k) acc[k] = 0.f;
           }
@@ -311,7 +326,8 @@ template <typename GT>
 __global__ __launch_bounds__(256) void seg_reduce_piece_finalize_kernel(
     const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
     const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
-    void *__restrict__ out, const float *__restrict__ scale, int pieces, int col0, int slice_w, int D) {
+    void *__restrict__ out, const float *__restrict__ scale, int pieces, int col0, int slice_w, int D,
+    int update) {
   constexpr int EV = 4, U = 4, kGroups = kWave / kPieceLanes;
   const int lane = lane_id();
   const int sub = lane & (kPieceLanes - 1), g = lane / kPieceLanes;
@@ -347,7 +363,16 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_finalize_kernel(
 #pragma unroll
       for (int k = 0; k < EV; ++k) acc[k] *= gs;
     }
-    if (g == 0 && d0 < D) store_vec<GT, EV>(out, static_cast<int64_t>(long_list[i]) * D + d0, acc);
+    if (g == 0 && d0 < D) {
+      const int64_t o = static_cast<int64_t>(long_list[i]) * D + d0;
+      if (update) {  // out is the weight matrix: subtract the (scaled) sum from it
+        float w[EV];
+        load_vec<GT, EV>(out, o, w);
+#pragma unroll
+        for (int k = 0; k < EV; ++k) acc[k] = w[k] - acc[k];
+      }
+      store_vec<GT, EV>(out, o, acc);
+    }
   }
 }
 

@@ -595,6 +595,75 @@ def _(indices, weight, vals, bias, target, need_dw=True):
             torch.empty_like(weight) if need_dw else weight.new_empty((0, weight.shape[1])))
 
 
+@torch.library.custom_op("flexsae_amd::hier_sgd_step", mutates_args=("weight",))
+def hier_sgd_step(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, target: Tensor,
+                  step: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+    """HierarchicalTopK training step with the plain-SGD decoder update fused in.
+
+    ``weight[f] -= step * dL/dW[f]`` for every latent f that ``indices`` touches, in place (fp32
+    arithmetic, one rounding to the weight's dtype); no dense gradient is formed and rows of
+    untouched latents are neither read nor written.  ``step`` is a 0-dim tensor: learning rate
+    times the upstream gradient of the loss.  Returns (loss, dvals, dbias) for a unit upstream
+    gradient and the weights as they were on entry: feed ``dvals`` to the encoder's backward
+    (``vals.backward(dvals * upstream)``) and apply ``dbias`` to the bias.
+    Takes the place of ``loss.backward(); torch.optim.SGD.step()`` for the decoder weight in a loop
+    written like reference example.py:76-77; with momentum or weight decay untouched rows change
+    too, and the dense gradient of ``triton_hierarchical_sae_loss`` is the interface to use.
+    ``weight`` must be contiguous and 16-byte aligned, D a multiple of 8 (16-bit) or 4 (fp32),
+    K <= 256."""
+    B, K, F, D = _validate(indices, weight, vals, bias, target)
+    if not weight.is_contiguous() or weight.data_ptr() % 16:
+        raise ValueError("hier_sgd_step updates weight in place: it must be contiguous and 16-byte aligned")
+    if not _train_supported(weight, K):
+        raise ValueError("hier_sgd_step needs D % 4 == 0 and K <= 256")
+    lib = _lib.load()
+    indices, vals, bias, target = (_prep(t) for t in (indices, vals, bias, target))
+    dev = weight.device
+    with torch.cuda.device(dev):
+        shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
+        p_size = 2 if weight.dtype == torch.bfloat16 else 4
+        slice_cols = _hier_slice_cols(B, K, p_size)
+        ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
+        dbias = torch.empty((D,), dtype=torch.float32, device=dev)
+        g = _grad_scalar(step, dev)
+        flag = _flag_for(dev)
+        cached = _pair_lookup(indices, F)
+        if cached is not None:
+            _pair_import(lib, shape, workspace, cached)
+        rc = lib.flexsae_hier_sgd_step(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
+                                       _ptr(target), _ptr(g), _ptr(loss), _ptr(dvals), _ptr(dbias),
+                                       _ptr(workspace), ws_bytes,
+                                       _lib.BWD_REUSE_PAIR_LIST if cached is not None else 0, _ptr(flag), _stream())
+        _lib.check(rc, "flexsae_hier_sgd_step")
+        if cached is None:
+            _pair_export(lib, shape, workspace, indices, F)
+        if _check_indices:
+            check_index_flag(dev)
+    return loss, dvals, dbias
+
+
+@hier_sgd_step.register_fake
+def _(indices, weight, vals, bias, target, step):
+    return (weight.new_empty((), dtype=torch.float32), vals.new_empty(vals.shape, dtype=torch.float32),
+            weight.new_empty((weight.shape[1],), dtype=torch.float32))
+
+
+def hierarchical_sae_sgd_step(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, target: Tensor,
+                              lr: float, grad_out=1.0) -> Tuple[Tensor, Tensor, Tensor]:
+    """``hier_sgd_step`` with a learning rate and an optional upstream gradient (float or 0-dim
+    tensor).  Runs without autograd: ``weight`` may be a leaf that requires grad; it is updated through
+    ``weight.data`` semantics (under ``torch.no_grad()``).  Returns (loss, dvals, dbias), unit upstream gradient."""
+    with torch.no_grad():
+        if isinstance(grad_out, Tensor):
+            step = (grad_out.detach().to(device=weight.device, dtype=torch.float32) * lr).reshape(())
+        else:
+            step = torch.tensor(float(lr) * float(grad_out), dtype=torch.float32, device=weight.device)
+        return hier_sgd_step(indices, weight, vals.detach(), bias.detach(), target, step)
+
+
 @torch.library.custom_op("flexsae_amd::scale_by", mutates_args=())
 def scale_by(x: Tensor, grad_out: Tensor) -> Tensor:
     """x * grad_out (a 0-dim scalar on the device), in x's dtype; replaces the reference's

@@ -208,6 +208,30 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, con
                          size_t workspace_bytes, int flags, int *status_flag, void *stream);
 
 /*
+ * HierarchicalTopK training step with the plain-SGD weight update fused in: the same pass as
+ * flexsae_hier_fwd_bwd, but the segment reduction, instead of writing a dense dW[F,D], subtracts
+ * step[0] * (unit-gradient row) from every weight row that the batch touches, in place, in the
+ * weight's own dtype (fp32 arithmetic, one rounding).  Rows of latents without pairs are neither
+ * read nor written, so the dense zero-fill, the dense dW and the optimizer's passes over dW and W
+ * are all gone.  `step` is a device fp32 scalar: learning rate times the upstream gradient of the
+ * loss.  loss, dvals and dbias are returned as by flexsae_hier_fwd_bwd (unit upstream gradient;
+ * dvals is what the encoder's backward needs, dbias the bias's update) and are computed from the
+ * weights as they were on entry: within a slice of columns every read of the weights precedes the
+ * reduction that updates that slice, and other slices touch other columns.
+ * Supported where flexsae_hier_fwd_bwd is and D is a multiple of 8 (16-bit weights) or 4 (fp32)
+ * with a 16-byte aligned weight matrix; otherwise FLEXSAE_ERR_UNSUPPORTED.  Workspace as for
+ * flexsae_hier_fwd_bwd; the only flag accepted is FLEXSAE_BWD_REUSE_PAIR_LIST.
+ * replaces: the dense dW of the backward (hierarchical_kernels.py:241-243, 294-297) together with
+ *           the optimizer pass that consumes it in a training loop written like reference
+ *           example.py:76-77 with torch.optim.SGD (no momentum, no weight decay: for those the
+ *           untouched rows change too, and the dense gradient is the right interface).
+ */
+int flexsae_hier_sgd_step(const flexsae_shape *shape, const int64_t *indices, void *weight,
+                          const void *vals, const void *bias, const void *target, const float *step,
+                          float *loss, float *dvals, float *dbias, void *workspace, size_t workspace_bytes,
+                          int flags, int *status_flag, void *stream);
+
+/*
  * dst[n] = src[n] * scale[0]  (same dtype in and out; `scale` is a device fp32 scalar).  dst may
  * be src (in place); then a scale of exactly 1 costs one empty launch.
  * replaces: the dW.mul_(grad) pass of HierarchicalSAELossFunction.backward

@@ -79,6 +79,22 @@ def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_
     return rc, loss, dW, dv, db
 
 
+def hier_sgd_step(indices, weight, vals, bias, target, step, flag=None, slice_cols=0):
+    """Training step with the SGD update of ``weight`` fused in (in place) -> (rc, loss, dvals, dbias)."""
+    lib = _lib.load()
+    sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
+    dev = weight.device
+    loss = torch.full((1,), float("nan"), dtype=torch.float32, device=dev)
+    dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
+    db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
+    nbytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    st = torch.tensor([step], dtype=torch.float32, device=dev)
+    rc = lib.flexsae_hier_sgd_step(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(bias), ptr(target),
+                                   ptr(st), ptr(loss), ptr(dv), ptr(db), ptr(ws), nbytes, 0, ptr(flag), stream())
+    return rc, loss, dv, db
+
+
 def scale(src, g, in_place=False):
     lib = _lib.load()
     dst = src if in_place else torch.full_like(src, float("nan"))

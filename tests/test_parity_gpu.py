@@ -148,6 +148,87 @@ def test_training_step_entry_point(shape, dtype):
     assert rel_err(dv.cpu(), dv4.cpu()) < 2e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["fp32", "bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(48, 32, 200, 768), (33, 128, 64, 2304), (9, 256, 700, 320), (64, 16, 1000, 8),
+                                   (40, 16, 200, 512), (50, 8, 333, 640), (16, 64, 9, 136)])
+def test_sgd_step_entry_point(shape, dtype):
+    """flexsae_hier_sgd_step through the C-ABI: W_new = W - step * dW of the oracle on the touched rows
+    (one rounding to the weight's dtype), untouched rows bit-identical to before, loss / dvals / dbias
+    bit-identical to flexsae_hier_fwd_bwd's (they come from the weights as they were on entry), for any
+    slice width."""
+    B, K, F, D = shape
+    _announce("sgd step abi", shape, dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=43)
+    idx, W, v, b, t = _to_dev(args)
+    step = 0.37
+    rc0, loss0, dW0, dv0, db0 = abi.hier_train(idx, W, v, b, t)
+    assert rc0 == 0
+    L, rW, rv, rb = oracle.loss_grads(oracle.HIER, *args, grad_out=1.0)
+    touched = torch.zeros(F, dtype=torch.bool)
+    touched[args[0].flatten()] = True
+    for cols in (0, 1 << 20):
+        Wn = W.clone()
+        rc, loss, dv, db = abi.hier_sgd_step(idx, Wn, v, b, t, step, slice_cols=cols)
+        torch.cuda.synchronize()
+        assert rc == 0, _lib.status_string(rc)
+        assert torch.equal(loss, loss0) and torch.equal(dv, dv0) and torch.equal(db, db0)
+        Wn = Wn.cpu()
+        assert torch.equal(Wn[~touched], args[1][~touched])
+        # the kernel's own fp32 gradient, rounded once: identical bits
+        expect = (W.float() - step * dW0).to(dtype).cpu()
+        if dtype == torch.float32:  # w - step*g may be contracted into one fused multiply-add
+            assert rel_err(Wn[touched], expect[touched]) < 1e-6
+        else:
+            assert (Wn[touched].float() - expect[touched].float()).abs().max() <= \
+                torch.finfo(dtype).eps * expect[touched].float().abs().max()
+        # and against the oracle: the update itself, not the updated weights (which it barely moves)
+        upd = (args[1].float()[touched] - Wn[touched].float()) / step
+        ref = torch.from_numpy(rW).float()[touched]
+        # rounding W_new to the weight's dtype quantises the recovered update at eps*|W|/step
+        quant = torch.finfo(dtype).eps * args[1].float().abs().max() / step
+        tol = 1e-4 if dtype == torch.float32 else 1e-2
+        assert (upd - ref).abs().max() <= tol * ref.abs().max() + quant
+
+
+def test_sgd_step_through_the_package():
+    """hierarchical_sae_sgd_step: one fused call equals loss.backward() + plain SGD on the decoder
+    weight; dvals and dbias are those of the autograd path; repeated steps lower the loss."""
+    args = make_inputs(64, 32, 500, 512, dtype=torch.float32, seed=44)
+    idx, W, v, b, t = _to_dev(args)
+    lr = 0.05
+    Wa = W.clone().requires_grad_()
+    va, ba = v.clone().requires_grad_(), b.clone().requires_grad_()
+    loss_a = flex.triton_hierarchical_sae_loss(idx, Wa, va, ba, t)
+    loss_a.backward()
+    W_sgd = (Wa.detach() - lr * Wa.grad)
+    Wf = W.clone().requires_grad_()   # a leaf that requires grad: updated in place without autograd
+    loss_f, dv, db = flex.hierarchical_sae_sgd_step(idx, Wf, v, b, t, lr)
+    torch.cuda.synchronize()
+    assert torch.equal(loss_f, loss_a.detach())
+    assert rel_err(Wf.detach().cpu(), W_sgd.cpu()) < 1e-6
+    assert torch.equal(dv, va.grad) and torch.equal(db, ba.grad)
+    losses = [loss_f.item()]
+    for _ in range(5):
+        l, _, _ = flex.hierarchical_sae_sgd_step(idx, Wf, v, b, t, 20.0)
+        losses.append(l.item())
+    assert all(x > y for x, y in zip(losses, losses[1:])), losses
+    # an upstream gradient scales the step
+    W2 = W.clone()
+    flex.hierarchical_sae_sgd_step(idx, W2, v, b, t, lr, grad_out=torch.tensor(2.0, device=DEV))
+    assert rel_err(W2.cpu(), (W - 2 * lr * Wa.grad).cpu()) < 1e-6
+    with pytest.raises(ValueError):
+        flex.hierarchical_sae_sgd_step(idx, W.t().contiguous().t(), v, b, t, lr)
+
+
+def test_sgd_step_unsupported_shapes():
+    idx, W, v, b, t = _to_dev(make_inputs(8, 8, 32, 12, dtype=torch.bfloat16, seed=3))  # D % 8 != 0 with 16-bit weights
+    rc, *_ = abi.hier_sgd_step(idx, W.clone(), v, b, t, 0.1)
+    assert rc == -2
+    idx, W, v, b, t = _to_dev(make_inputs(8, 8, 32, 12, seed=3))  # fp32: a multiple of 4 is enough
+    rc, *_ = abi.hier_sgd_step(idx, W.clone(), v, b, t, 0.1)
+    assert rc == 0
+
+
 def test_training_step_unsupported_shapes_and_scale():
     idx, W, v, b, t = _to_dev(make_inputs(8, 8, 32, 6, seed=3))  # D % 4 != 0
     rc, *_ = abi.hier_train(idx, W, v, b, t)
@@ -694,6 +775,7 @@ def test_opcheck_of_every_op_with_all_checks():
     torch.library.opcheck(ops.hier_finish, (g, idx, W, v, stage))
     torch.library.opcheck(ops.scale_by, (W, g))
     torch.library.opcheck(ops.scale_, (W.clone(), g))
+    torch.library.opcheck(ops.hier_sgd_step, (idx, W.clone(), v, b, t, g))  # mutates its weight argument
 
 
 @pytest.mark.parametrize("mode", ["hier", "topk"])
