@@ -526,8 +526,9 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
     int pps_shift = -1;  // log2(pps) when pps is a power of two
     for (int sh = 0; sh < 16; ++sh)
       if (pps == (1 << sh)) pps_shift = sh;
-    // latents per group of lanes: several where latents have few rows on average
-    const int per_group = n_pairs <= 2 * F ? 4 : n_pairs <= 4 * F ? 2 : 1;
+    // latents per group of lanes: four where most latents have no or few rows (with four rows per
+    // latent on average the bookkeeping already costs more than the shorter launch saves)
+    const int per_group = n_pairs <= 2 * F ? 4 : 1;
 #define FLEXSAE_PIECE_REDUCE(G)                                                                                    \
   hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_PIECE_U, G>),                                        \
                      dim3(kLongBlocks + static_cast<unsigned>(ceil_div(ceil_div(F, G) * pps, kBlock / kPieceLanes))), \
@@ -535,8 +536,6 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
                      F, kLongBlocks, pps, pps_shift, col0, sw, D, update)
     if (per_group == 4) {
       FLEXSAE_PIECE_REDUCE(4);
-    } else if (per_group == 2) {
-      FLEXSAE_PIECE_REDUCE(2);
     } else {
       FLEXSAE_PIECE_REDUCE(1);
     }
@@ -625,8 +624,16 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
 #undef FLEXSAE_SWEEP
     }
     if (!do_reduce) continue;
+    // Pieces where the slice is not made of whole reduction tiles, where most latents are empty
+    // (four latents per group of lanes), for the in-place update, and where a slice of
+    // contributions is about the size of the memory-side cache (measured 1 % faster there); else one
+    // wavefront per (latent, reduction tile), which wastes no load slots on the unequal row counts
+    // of the four latents a wavefront would otherwise share (4 % faster on slices read from HBM).
+    const bool cache_sized = static_cast<size_t>(s->B * s->K) * static_cast<size_t>(sw) * pl.p_size <= (size_t{384} << 20);
+    const bool by_pieces =
+        piece != 0 && (update || cols % pl.tile != 0 || s->B * s->K <= 2 * s->F || cache_sized);
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
-                                   static_cast<int>(col0), sw, D, st, piece, cols, s->B * s->K, update);
+                                   static_cast<int>(col0), sw, D, st, by_pieces ? piece : 0, cols, s->B * s->K, update);
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only

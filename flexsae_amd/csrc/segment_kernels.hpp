@@ -39,6 +39,38 @@ __device__ __forceinline__ void accumulate_rows(const void *__restrict__ X, int6
   }
 }
 
+// The same sum in the order of the reduction by pieces (below), so that both reductions give the
+// same bits for long latents: four running sums, row j goes to sum j % 4, combined as
+// (s0 + s1) + (s2 + s3).
+template <typename PT, int VEC, int U, bool NT = false>
+__device__ __forceinline__ void accumulate_rows_by4(const void *__restrict__ X, int64_t r0, int n,
+                                                    int64_t ld, int pc, float (&acc)[VEC]) {
+  static_assert(U % 4 == 0, "rows are dealt to four sums");
+  float part[4][VEC];
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) part[g][i] = 0.f;
+  for (int j = 0; j < n; j += U) {
+    raw_vec_t<PT, VEC> raw[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (j + u < n) raw[u] = load_raw<PT, VEC, NT>(X, (r0 + j + u) * ld + pc);  // uniform
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (j + u < n) {  // uniform
+        float x[VEC];
+        unpack_raw<PT, VEC>(raw[u], x);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) part[u & 3][i] += x[i];
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) acc[i] = (part[0][i] + part[1][i]) + (part[2][i] + part[3][i]);
+}
+
 // Decode work item `chunk` of the long-latent work list: which latent, which rows.
 struct LongChunk {
   uint32_t long_slot;
@@ -115,7 +147,7 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-    accumulate_rows<PT, VEC, 8, FLEXSAE_REDUCE_NT>(P, c.s0, static_cast<int>(c.s1 - c.s0), slice_w, pc, acc);
+    accumulate_rows_by4<PT, VEC, 8, FLEXSAE_REDUCE_NT>(P, c.s0, static_cast<int>(c.s1 - c.s0), slice_w, pc, acc);
     store_vec<float, VEC>(partial, static_cast<int64_t>(chunk) * slice_w + pc, acc);
   }
 }
@@ -396,7 +428,7 @@ __global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
     float acc[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
-    accumulate_rows<float, VEC, U>(partial, c0, static_cast<int>(c1 - c0), slice_w, pc, acc);
+    accumulate_rows_by4<float, VEC, U>(partial, c0, static_cast<int>(c1 - c0), slice_w, pc, acc);
     if (scale) {
       const float g = scale[0];
 #pragma unroll
