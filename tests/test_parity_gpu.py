@@ -124,7 +124,7 @@ def test_training_step_entry_point(shape, dtype):
     """flexsae_hier_fwd_bwd through the C-ABI: loss and unit-gradient gradients in one pass, for
     K that are not powers of two (up to 256, where a wavefront keeps part of the row pieces in
     accumulation registers), D that are not whole tiles, hot latents (F tiny), and between one and
-    four pairs per latent on average (the reduction then serves two or four latents per group of lanes)."""
+    four pairs per latent on average (with at most two the reduction serves four latents per group of lanes)."""
     B, K, F, D = shape
     _announce("train abi", shape, dtype)
     args = make_inputs(B, K, F, D, dtype=dtype, seed=41)
