@@ -452,19 +452,41 @@ struct TrainArgs {
 // largest K the training-step kernel holds in registers
 inline bool train_supported(const flexsae_shape *s) { return s->D % 4 == 0 && s->K <= 256; }
 
+// Row pieces the training-step kernel keeps in the LDS instead of registers (one dword per lane
+// and row: 16-bit weights with two columns per lane, fp32 with one), chosen so that one more
+// wavefront fits each SIMD: 256 steps 216 instead of 276 registers (two wavefronts instead of one,
+// 16 KB of LDS each), 128 steps 120 instead of 152 (four instead of three, 8 KB each), 64 steps 72
+// instead of 88.
+#ifndef FLEXSAE_LDS_256
+#define FLEXSAE_LDS_256 64
+#endif
+#ifndef FLEXSAE_LDS_128
+#define FLEXSAE_LDS_128 32
+#endif
+#ifndef FLEXSAE_LDS_64
+#define FLEXSAE_LDS_64 16
+#endif
+template <typename WT, int KMAX, int VEC>
+constexpr int train_lds_rows() {
+  if (VEC * sizeof(typename Traits<WT>::store_t) != 4) return 0;
+  return KMAX == 256 ? FLEXSAE_LDS_256 : KMAX == 128 ? FLEXSAE_LDS_128 : KMAX == 64 ? FLEXSAE_LDS_64 : 0;
+}
+
 template <typename WT, typename PT, int KMAX, int VEC = 2>
 void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
                          const void *weight, const void *vals, float coef, const uint32_t *slot, void *P,
                          float *dvals, float *s_final, int d_pad, float *loss_partial, int *status_flag,
                          int64_t cols, int col0, int slice_w, hipStream_t st) {
+  constexpr int LDSROWS = train_lds_rows<WT, KMAX, VEC>();
   const int64_t n_items = s->B * (cols / (kWave * VEC));
-  // K == KMAX (the usual powers of two) runs the variant without per-step bound tests
+  // K == KMAX (the usual powers of two) runs the variant without per-step bound tests, part of its
+  // row pieces in the LDS
   const bool stream = slice_w >= d_pad;  // all of P in one launch: streaming stores
   const auto kernel = s->K == KMAX
-                          ? (stream ? hier_train_kernel<WT, PT, KMAX, true, true, VEC>
-                                    : hier_train_kernel<WT, PT, KMAX, true, false, VEC>)
-                          : (stream ? hier_train_kernel<WT, PT, KMAX, false, true, VEC>
-                                    : hier_train_kernel<WT, PT, KMAX, false, false, VEC>);
+                          ? (stream ? hier_train_kernel<WT, PT, KMAX, true, true, VEC, LDSROWS>
+                                    : hier_train_kernel<WT, PT, KMAX, true, false, VEC, LDSROWS>)
+                          : (stream ? hier_train_kernel<WT, PT, KMAX, false, true, VEC, 0>
+                                    : hier_train_kernel<WT, PT, KMAX, false, false, VEC, 0>);
   hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
                      indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
                      coef, slot, P, dvals, s_final, d_pad, loss_partial, status_flag, n_items, s->B, col0,

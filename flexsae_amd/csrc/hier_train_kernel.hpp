@@ -60,11 +60,18 @@ struct RowPiece<f16_t, 2> {
 // Row gathers and contribution stores go through per-row buffer descriptors: their address
 // arithmetic runs on the scalar unit, lanes beyond column D read zeros (so their dot products
 // vanish), and what such lanes store lands in the padding columns of P, which nobody reads.
+// LDSROWS (FULL variants only): the first LDSROWS row pieces are loaded straight into the LDS
+// (buffer load with the LDS as destination, one dword per lane) instead of registers, which buys
+// one more wavefront per SIMD: 120 instead of 152 registers at 128 steps (four wavefronts, 8 KB of
+// LDS each), 216 instead of 276 at 256 steps (two wavefronts, 16 KB each).  Both walks read them
+// back with plain LDS loads.  bias - target is fetched before the gathers are issued: the memory
+// counter retires in order, so anything issued after them can only be waited for together with
+// all of them, and the forward walk could not start while rows are still arriving.
 // STREAM: the contributions are stored with the non-temporal hint.  That is the faster choice
 // when all of P is written before any of it is read back (it is far larger than the caches);
 // when P is one slice that the reduction reads right after this launch, plain stores leave part
 // of it in the memory-side cache and the pair of launches is faster.
-template <typename WT, typename PT, int KMAX, bool FULL, bool STREAM, int VEC>
+template <typename WT, typename PT, int KMAX, bool FULL, bool STREAM, int VEC, int LDSROWS = 0>
 __global__ __launch_bounds__(256) void hier_train_kernel(
     const int64_t *__restrict__ indices, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
@@ -77,6 +84,10 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   using S_t = typename Traits<WT>::store_t;
   constexpr int KC = (KMAX + kWave - 1) / kWave;  // 64-step chunks held per lane
   static_assert(KMAX % 8 == 0, "KMAX must be a multiple of 8");
+  static_assert(LDSROWS == 0 || (sizeof(raw_t) == 4 && LDSROWS <= KMAX && FULL), "LDS rows hold one dword per lane");
+  // the first LDSROWS row pieces live in the LDS (loaded straight into it), the rest in registers
+  __shared__ uint32_t lds_rows[LDSROWS > 0 ? (256 / kWave) * LDSROWS * kWave : 1];
+  uint32_t *const my_lds = lds_rows + wave_in_block() * (LDSROWS * kWave);
   const int lane = lane_id();
   const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
   if (item >= n_items) return;  // uniform per wavefront
@@ -117,6 +128,17 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     my_row[c] = static_cast<int>(idx);
   }
 
+  // bias - target first: the memory counter retires in order, so a load issued after the gathers
+  // could only be waited for together with all of them
+  float e[VEC], tt[VEC], acc[VEC];
+  load_vec_dyn<WT, VEC>(bias, bias_dtype, dsafe, e);
+  load_vec_dyn<WT, VEC>(target, target_dtype, b * D + dsafe, tt);
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    e[i] -= tt[i];
+    acc[i] = 0.f;
+  }
+
   // all gathers at once
   raw_t raw[KMAX];
   const uint32_t w_row_bytes = static_cast<uint32_t>(D) * sizeof(S_t);
@@ -127,19 +149,29 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     for (int k = 0; k < KMAX; ++k) {
       if (FULL || k < kb) {  // uniform
         const uint32_t row = static_cast<uint32_t>(bcast_i32(my_row[k / kWave], k % kWave));
+        if constexpr (LDSROWS > 0) {
+          if (k < LDSROWS) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                row_descriptor(weight, row, w_row_bytes),
+                (__attribute__((address_space(3))) void *)(my_lds + k * kWave),
+                4, w_lane_bytes, 0, 0, 0);
+            continue;
+          }
+        }
         const auto dw = descriptor_load<sizeof(raw_t)>(row_descriptor(weight, row, w_row_bytes), w_lane_bytes);
         __builtin_memcpy(&raw[k], &dw, sizeof(raw_t));
       }
     }
   }
 
-  float e[VEC], tt[VEC], acc[VEC];
-  load_vec_dyn<WT, VEC>(bias, bias_dtype, dsafe, e);
-  load_vec_dyn<WT, VEC>(target, target_dtype, b * D + dsafe, tt);
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    e[i] -= tt[i];
-    acc[i] = 0.f;
+
+  if constexpr (LDSROWS > 0) {
+    // The compiler does not order LDS reads after the loads that fill the LDS.  The memory counter
+    // retires in order (and holds at most 63), so once no more than (loads issued - LDSROWS) are
+    // outstanding the first LDSROWS have landed; the memory clobber keeps the reads below.
+    static_assert(FULL, "the wait below counts on all KMAX loads having been issued");
+    constexpr int kLeft = KMAX - LDSROWS < 63 ? KMAX - LDSROWS : 63;
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLeft) : "memory");
   }
 
   // forward walk
@@ -149,7 +181,18 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     if (FULL || k < kb_fwd) {  // uniform
       const float v = bcast_f32(my_val[k / kWave], k % kWave);
       float w[VEC];
-      Piece::unpack(raw[k], w);
+      if constexpr (LDSROWS > 0) {
+        if (k < LDSROWS) {
+          raw_t rk;
+          const uint32_t x = my_lds[k * kWave + lane];
+          __builtin_memcpy(&rk, &x, sizeof(raw_t));
+          Piece::unpack(rk, w);
+        } else {
+          Piece::unpack(raw[k], w);
+        }
+      } else {
+        Piece::unpack(raw[k], w);
+      }
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         e[i] = fmaf(w[i], v, e[i]);
@@ -184,7 +227,17 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
           const uint32_t prow = static_cast<uint32_t>(bcast_i32(my_slot[k / kWave], k % kWave));
           // Without this the compiler reuses the unpacked values of the forward walk, which
           // doubles the registers held across the two walks; re-unpacking costs one op per value.
-          raw_t rk = raw[k];
+          raw_t rk;
+          if constexpr (LDSROWS > 0) {
+            if (k < LDSROWS) {
+              const uint32_t x = my_lds[k * kWave + lane];
+              __builtin_memcpy(&rk, &x, sizeof(raw_t));
+            } else {
+              rk = raw[k];
+            }
+          } else {
+            rk = raw[k];
+          }
           Piece::launder(rk);
           float w[VEC], contrib[VEC];
           Piece::unpack(rk, w);

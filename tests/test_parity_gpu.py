@@ -288,10 +288,12 @@ def test_fused_training_backward_twice_and_no_grad(stage):
 
 @pytest.mark.parametrize("mode", ["hier", "topk"])
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (3, 5, 7, 9), (5, 3, 11, 70), (2, 65, 40, 130),
-                                   (7, 130, 300, 200), (4, 24, 50, 1000), (33, 12, 17, 2304)])
+                                   (7, 130, 300, 200), (4, 24, 50, 1000), (33, 12, 17, 2304), (3, 300, 900, 136),
+                                   (2, 512, 4096, 64)])
 def test_odd_shapes_fp32(mode, shape):
     """Sizes the reference's static asserts reject: K not a power of two, K > 64 with a ragged
-    last group, D not a multiple of 64 (nor of the vector width), B not a multiple of 16."""
+    last group, D not a multiple of 64 (nor of the vector width), B not a multiple of 16; rows of
+    more than 256 steps (forward + sliced backward instead of the training-step kernel)."""
     B, K, F, D = shape
     _announce("odd", mode, shape)
     args = make_inputs(B, K, F, D, seed=B + K + F + D)
