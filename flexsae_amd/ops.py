@@ -175,11 +175,6 @@ topk_fwd.register_fake(_fwd_fake)
 # Scratch the hierarchical backward may use for the per-pair contributions of one slice of D
 # columns.  More scratch = wider slices = fewer passes; 0 selects the atomic single-pass fallback.
 _hier_scratch_bytes = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
-# Rows of more than 128 steps run one wavefront per SIMD (each keeps up to 256 row pieces in
-# registers), so every launch ends in a long tail and few wide slices beat many narrow ones:
-# unless a scratch size was set explicitly, such problems may use eight times the default.
-_hier_scratch_explicit = "FLEXSAE_HIER_SCRATCH_MB" in os.environ
-_LONG_ROW_SCRATCH_FACTOR = 8
 
 
 # Narrowest slice the scratch budget may lead to on its own: slices below 256 columns run slower
@@ -196,8 +191,6 @@ def set_hier_min_slice_cols(cols: int) -> None:
 
 
 def _hier_scratch_budget(K: int) -> int:
-    if K > 128 and not _hier_scratch_explicit:
-        return _hier_scratch_bytes * _LONG_ROW_SCRATCH_FACTOR
     return _hier_scratch_bytes
 
 
@@ -209,15 +202,10 @@ def set_hier_scratch_bytes(nbytes) -> None:
     """Upper bound on the scratch of the hierarchical backward (bytes).  0 = use the atomic
     scatter fallback, which needs no scratch but an fp32 [F,D] accumulator.  The default (256 MiB)
     is the size at which one slice of contributions stays in the memory-side cache between the
-    sweep that writes it and the reduction that reads it; wider slices run slower, not faster --
-    except for rows of more than 128 steps, which get eight times the default unless a size is set
-    here or through FLEXSAE_HIER_SCRATCH_MB."""
-    global _hier_scratch_bytes, _hier_scratch_explicit
-    if nbytes is None:  # back to the default rule
-        _hier_scratch_bytes, _hier_scratch_explicit = 256 << 20, False
-        return
-    _hier_scratch_bytes = int(nbytes)
-    _hier_scratch_explicit = True
+    sweep that writes it and the reduction that reads it; wider slices run slower, not faster.
+    ``None`` restores the default."""
+    global _hier_scratch_bytes
+    _hier_scratch_bytes = (256 << 20) if nbytes is None else int(nbytes)
 
 
 # Memory the fused training step may hold between forward and backward: all B*K*D per-pair
