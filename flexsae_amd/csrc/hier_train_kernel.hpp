@@ -218,6 +218,16 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   for (int k8 = KMAX - 8; k8 >= 0; k8 -= 8) {
     if (FULL || k8 < kb_rev) {  // uniform
       float dots[8];
+      raw_t from_lds[8];  // the block's LDS rows, fetched together ahead of their use
+      if constexpr (LDSROWS > 0) {
+        if (k8 < LDSROWS) {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const uint32_t x = my_lds[(k8 + u) * kWave + lane];
+            __builtin_memcpy(&from_lds[u], &x, sizeof(raw_t));
+          }
+        }
+      }
 #pragma unroll
       for (int u = 7; u >= 0; --u) {
         const int k = k8 + u;
@@ -230,8 +240,7 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
           raw_t rk;
           if constexpr (LDSROWS > 0) {
             if (k < LDSROWS) {
-              const uint32_t x = my_lds[k * kWave + lane];
-              __builtin_memcpy(&rk, &x, sizeof(raw_t));
+              rk = from_lds[u];
             } else {
               rk = raw[k];
             }
