@@ -511,7 +511,7 @@ void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const in
   } else if constexpr (sizeof(typename Traits<WT>::store_t) == 2) {
     if (s->K <= 128) {
       FLEXSAE_TRAIN(128);
-    } else {  // 129..256 steps: one wavefront per SIMD, part of the row pieces in accumulation registers
+    } else {  // 129..256 steps: two wavefronts per SIMD with 64 rows in the LDS (K = 256), else one
       FLEXSAE_TRAIN(256);
     }
   } else if (s->K <= 128) {  // fp32 rows of 65..128 steps: one column per lane

@@ -175,8 +175,8 @@ int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const v
  * the real one afterwards (flexsae_scale for dW; dvals/dbias are small).  Same workspace, same
  * slicing and the same segment reduction as flexsae_hier_bwd (use
  * flexsae_hier_bwd_workspace_bytes).
- * Supported when D % 4 == 0 and K <= 256 (the row pieces of a tile are kept in registers; beyond
- * 128 steps a wavefront has a SIMD's register file to itself):
+ * Supported when D % 4 == 0 and K <= 256 (the row pieces of a tile are kept on chip: in registers
+ * and, for K = 64, 128 or 256, a quarter of them in the LDS):
  * flexsae_hier_fwd_bwd_supported() tells; otherwise FLEXSAE_ERR_UNSUPPORTED (use
  * flexsae_hier_fwd + flexsae_hier_bwd).
  * replaces: the forward and backward kernels and launchers together

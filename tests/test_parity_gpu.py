@@ -122,8 +122,8 @@ def test_reference_matrix_without_fused_training(B, K, F, D, dtype):
                                    (12, 200, 3000, 72), (40, 16, 200, 512), (50, 8, 333, 640)])
 def test_training_step_entry_point(shape, dtype):
     """flexsae_hier_fwd_bwd through the C-ABI: loss and unit-gradient gradients in one pass, for
-    K that are not powers of two (up to 256, where a wavefront keeps part of the row pieces in
-    accumulation registers), D that are not whole tiles, hot latents (F tiny), and between one and
+    K that are and are not powers of two, up to 256 (the kernel variants with and without row
+    pieces in the LDS), D that are not whole tiles, hot latents (F tiny), and between one and
     four pairs per latent on average (with at most two the reduction serves four latents per group of lanes)."""
     B, K, F, D = shape
     _announce("train abi", shape, dtype)
