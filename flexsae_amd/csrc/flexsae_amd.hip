@@ -373,6 +373,13 @@ inline int64_t train_tile_cols(const flexsae_shape *s) {
 
 // ---- two-phase hierarchical backward: workspace plan -----------------------------------
 
+constexpr int kClsStride = 80;  // slots per counter array of the class list
+static_assert(kSegClasses + 1 <= kClsStride, "a counter array holds one slot per class and the total");
+
+// Most latents without a pair, the rest with few: the reduction by pieces then works from the list
+// of latents ordered by row count and the rows of latents without pairs are zeroed in one pass.
+inline bool sparse_latents(const flexsae_shape *s) { return s->B * s->K <= 2 * s->F; }
+
 struct HierBwdPlan {
   int vec;                 // columns per lane
   int tile;                // 64 * vec columns per wavefront
@@ -381,7 +388,7 @@ struct HierBwdPlan {
   size_t n_pairs;          // B * K
   size_t n_rows;           // B
   size_t n_partial_rows;   // upper bound on the number of 64-pair chunks of long latents
-  size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_sfinal, off_colsum, off_loss, off_dvpart, off_partial;  // per-slice buffers follow
+  size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_cls, off_cls_list, off_sfinal, off_colsum, off_loss, off_dvpart, off_partial;  // per-slice buffers follow
   size_t n_loss_partials;  // training-step kernel: one per (tile of 64 or 128 columns, row)
   size_t fixed_bytes;      // everything that does not depend on the slice width
 };
@@ -406,6 +413,12 @@ HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
   off += flexsae_csr_workspace_bytes(s->B, s->K, s->F);
   p.off_chunk = off;
   off += round_up((p.n_pairs / 65 + 2) * 4, kAlign);
+  // latents ordered by row count (sparse shapes, see seg_class_scatter_kernel): three counter
+  // arrays of kClsStride slots (histogram, cursors, first entry of every class) and the list
+  p.off_cls = off;
+  off += round_up(3 * static_cast<size_t>(kClsStride) * 4, kAlign);
+  p.off_cls_list = off;
+  off += round_up(static_cast<size_t>(s->F) * 4, kAlign);
   p.off_sfinal = off;  // S_{b,0} of every row, [B, d_pad] fp32: dbias is its column sum
   off += round_up(p.n_rows * static_cast<size_t>(p.d_pad) * 4, kAlign);
   p.off_colsum = off;  // partial column sums, [ceil(B/64), D] fp32
@@ -542,24 +555,28 @@ template <typename PT, typename GT, int VEC>
 void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc, const uint32_t *chunk_begin,
                        const void *P, float *partial, void *dW, const float *dw_scale, int64_t F, int tps,
                        int col0, int sw, int D, hipStream_t st, int piece_cols = 0, int64_t cols = 0, int64_t n_pairs = 0,
-                       int update = 0) {
+                       int update = 0, const uint32_t *cls_begin = nullptr, const uint32_t *cls_list = nullptr) {
   if (piece_cols > 0) {  // 256-byte pieces, sixteen lanes each
     const int pps = static_cast<int>(cols / piece_cols);
     int pps_shift = -1;  // log2(pps) when pps is a power of two
     for (int sh = 0; sh < 16; ++sh)
       if (pps == (1 << sh)) pps_shift = sh;
-    // latents per group of lanes: four where most latents have no or few rows (with four rows per
-    // latent on average the bookkeeping already costs more than the shorter launch saves)
-    const int per_group = n_pairs <= 2 * F ? 4 : 1;
-#define FLEXSAE_PIECE_REDUCE(G)                                                                                    \
+    // latents per group of lanes: four, taken from the list ordered by row count, where most latents
+    // have no or few rows (with four rows per latent on average the bookkeeping already costs more
+    // than the shorter launch saves); the list holds at most min(F, pairs) latents with rows
+#define FLEXSAE_PIECE_REDUCE(G, N_ITEMS, CLS_LIST, CLS_BEGIN)                                                      \
   hipLaunchKernelGGL((seg_reduce_piece_kernel<PT, GT, FLEXSAE_PIECE_U, G>),                                        \
-                     dim3(kLongBlocks + static_cast<unsigned>(ceil_div(ceil_div(F, G) * pps, kBlock / kPieceLanes))), \
+                     dim3(kLongBlocks +                                                                            \
+                          static_cast<unsigned>(ceil_div((N_ITEMS) * pps, kBlock / kPieceLanes))),             \
                      dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, \
-                     F, kLongBlocks, pps, pps_shift, col0, sw, D, update)
-    if (per_group == 4) {
-      FLEXSAE_PIECE_REDUCE(4);
+                     F, kLongBlocks, pps, pps_shift, col0, sw, D, update, CLS_LIST, CLS_BEGIN)
+    if (cls_list) {
+      // work items of the list: one per latent with kSegBigRows rows or more, one per four others
+      const int64_t n_listed_max = F < n_pairs ? F : n_pairs;
+      const int64_t n_items_max = n_pairs / kSegBigRows + ceil_div(n_listed_max, 4) + 1;
+      FLEXSAE_PIECE_REDUCE(4, n_items_max, cls_list, cls_begin);
     } else {
-      FLEXSAE_PIECE_REDUCE(1);
+      FLEXSAE_PIECE_REDUCE(1, F, static_cast<const uint32_t *>(nullptr), static_cast<const uint32_t *>(nullptr));
     }
 #undef FLEXSAE_PIECE_REDUCE
     // the chunk partials of hot latents are combined per 64-column piece
@@ -622,6 +639,14 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   int sweep_vec = VEC;
   const int min_sweep_vec = static_cast<int>((pl.tile < train_tile_cols(s) ? pl.tile : train_tile_cols(s)) / kWave);
   while (sweep_vec > 1 && sweep_vec > min_sweep_vec && s->B * (slice_w / (kWave * sweep_vec)) < 6144) sweep_vec >>= 1;
+  // Sparse shapes reduce every slice by pieces from the list of latents ordered by row count; the
+  // rows of latents without pairs are zeroed here, whole rows in one pass (the in-place update leaves
+  // them alone).
+  const bool sparse = piece != 0 && sparse_latents(s);
+  const uint32_t *cls_begin = reinterpret_cast<const uint32_t *>(ws + pl.off_cls) + 2 * kClsStride;
+  const uint32_t *cls_list = reinterpret_cast<const uint32_t *>(ws + pl.off_cls_list);
+  if (sparse && do_reduce && !update)
+    hipLaunchKernelGGL((seg_zero_rows_kernel<PT, GT>), dim3(2048), dim3(kBlock), 0, st, cls_begin, cls_list, dW, D);
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (d_used - col0) < slice_w ? (d_used - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
@@ -655,7 +680,8 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     const bool by_pieces =
         piece != 0 && (update || cols % pl.tile != 0 || s->B * s->K <= 2 * s->F || cache_sized);
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
-                                   static_cast<int>(col0), sw, D, st, by_pieces ? piece : 0, cols, s->B * s->K, update);
+                                   static_cast<int>(col0), sw, D, st, by_pieces ? piece : 0, cols, s->B * s->K, update,
+                                   sparse ? cls_begin : nullptr, sparse ? cls_list : nullptr);
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
@@ -711,6 +737,22 @@ void launch_hier_slices_w(const flexsae_shape *s, const HierBwdPlan &pl, int64_t
       launch_hier_slices_g<f16_t, float, VEC>(s, pl, slice_w, indices, weight, vals, resid, grad_out,
                                               coef, dW, dW_dtype, dvals, dbias, ws, flags, status_flag, st, train, piece);
   }
+}
+
+// What follows the pair list in a hierarchical workspace: the chunk table of the hot latents and, for
+// sparse shapes, the list of latents ordered by row count.
+void finish_pair_list(const flexsae_shape *s, const HierBwdPlan &pl, uint8_t *ws, const uint32_t *begin,
+                      const CsrScratch &sc, hipStream_t st) {
+  uint32_t *cls = reinterpret_cast<uint32_t *>(ws + pl.off_cls);
+  const bool sparse = sparse_latents(s);
+  hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count, sc.long_list,
+                     reinterpret_cast<uint32_t *>(ws + pl.off_chunk), sparse ? cls : static_cast<uint32_t *>(nullptr),
+                     2 * kClsStride);
+  if (!sparse) return;
+  hipLaunchKernelGGL(seg_class_hist_kernel, dim3(grid_for(s->F, 256, 1024)), dim3(256), 0, st, begin, s->F, cls);
+  hipLaunchKernelGGL(seg_class_scatter_kernel, dim3(static_cast<unsigned>(ceil_div(s->F, 256 * kClassPerThread))),
+                     dim3(256), 0, st, begin, s->F, cls, cls + kClsStride, cls + 2 * kClsStride,
+                     reinterpret_cast<uint32_t *>(ws + pl.off_cls_list));
 }
 
 // ---- TopK backward: workspace plan and slice loop ---------------------------------------
@@ -994,8 +1036,7 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
     csr_build_launch(indices, s->B, s->K, s->F, begin, map, reinterpret_cast<uint32_t *>(ws + pl.off_slot), sc,
                      status_flag, st);
-    hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
-                       sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+    finish_pair_list(s, pl, ws, begin, sc, st);
   }
   const float coef = static_cast<float>(
       2.0 / (static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D)));
@@ -1047,8 +1088,7 @@ int flexsae_hier_import_pair_list(const flexsae_shape *s, const uint32_t *begin,
   hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, sc.long_count, static_cast<int64_t>(1), 0u);
   hipLaunchKernelGGL(seg_find_long_kernel, dim3(grid_for(s->F, 256, 2048)), dim3(256), 0, st, ws_begin, s->F,
                      sc.long_count, sc.long_list);
-  hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, ws_begin, sc.long_count, sc.long_list,
-                     reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+  finish_pair_list(s, pl, ws, ws_begin, sc, st);
   return launch_status();
 }
 
@@ -1106,8 +1146,7 @@ int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
     csr_build_launch(indices, s->B, s->K, s->F, begin, map, reinterpret_cast<uint32_t *>(ws + pl.off_slot), sc,
                      status_flag, st);
-    hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count,
-                       sc.long_list, reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+    finish_pair_list(s, pl, ws, begin, sc, st);
   }
   const double count = static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D);
   const float coef = static_cast<float>(2.0 / count);
@@ -1230,7 +1269,7 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
   hipLaunchKernelGGL(seg_find_long_kernel, dim3(grid_for(s->F, 256, 2048)), dim3(256), 0, st, begin, s->F,
                      long_count, long_list);
   hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, long_count, long_list,
-                     reinterpret_cast<uint32_t *>(ws + pl.off_chunk));
+                     reinterpret_cast<uint32_t *>(ws + pl.off_chunk), static_cast<uint32_t *>(nullptr), 0);
   const float coef =
       static_cast<float>(2.0 / (static_cast<double>(s->B) * static_cast<double>(s->D)));
   // per-pair records and, for bf16 weights, the bf16 copy of the residual: one launch

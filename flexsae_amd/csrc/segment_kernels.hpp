@@ -14,6 +14,8 @@
 namespace flexsae {
 
 constexpr int kSegChunk = 64;  // rows per chunk; groups longer than this count as "long"
+constexpr int kSegClasses = kSegChunk + 1;  // row counts 0..kSegChunk of the list ordered by row count (below)
+constexpr int kSegBigRows = 9;  // latents with at least this many rows get a group of lanes to themselves there
 
 // acc += sum of rows [r0, r0+n) of X (row stride `ld` elements) over the lane's VEC columns at pc.
 // Rows are fetched up to U at a time; n is uniform over the wavefront, so the tests around the
@@ -159,7 +161,9 @@ __global__ __launch_bounds__(256) void seg_reduce_kernel(
 // and this one.  The four latents (or pieces) of a wavefront have different row counts: the loop
 // runs to the longest, loads beyond a group's own count are masked off.  Work order: pieces of a
 // latent adjacent, latents ascending, so the launch still reads P front to back.  G > 1: a group
-// serves G consecutive latents (chosen by the caller where latents have few rows on average).
+// serves G latents taken from the list ordered by row count (cls_list / cls_begin, see
+// seg_class_scatter_kernel; chosen by the caller where most latents have no or few rows), and
+// latents without rows are not written here.
 constexpr int kPieceLanes = 16;
 constexpr int kPieceBytes = kPieceLanes * 16;
 
@@ -169,7 +173,8 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
     const uint32_t *__restrict__ long_list, const uint32_t *__restrict__ chunk_begin,
     const void *__restrict__ P, float *__restrict__ partial, void *__restrict__ out,
     const float *__restrict__ scale, int64_t F, unsigned n_long_blocks, int pps, int pps_shift, int col0,
-    int slice_w, int D, int update) {
+    int slice_w, int D, int update, const uint32_t *__restrict__ cls_list,
+    const uint32_t *__restrict__ cls_begin) {
   using S = typename Traits<PT>::store_t;
   constexpr int EV = 16 / static_cast<int>(sizeof(S));  // columns per lane
   constexpr int kGroupsPerBlock = 256 / kPieceLanes;
@@ -254,48 +259,58 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
       }
       if (mine && !(update && n == 0)) emit(f, d0, acc);
     } else {
-      // Few rows per latent: a launch of one latent per group is a train of short-lived wavefronts,
-      // each waiting for two dependent round trips (begin[], then the rows).  Here a group serves G
-      // consecutive latents: their rows are adjacent in P (apart from those of a long latent in
-      // between), so they are fetched U at a time regardless of where one latent ends and the next
-      // begins, and a latent's sum is stored when its last row has been added.  The order of the
-      // additions of a latent is the same as with G = 1.
-      const int64_t f0 = fb * G;
-      uint32_t bv = 0;  // lane j of the group holds begin[f0 + j], j <= G
-      if (f0 < F && sub <= G) bv = begin[f0 + sub < F ? f0 + sub : F];
-      uint32_t c[G + 1], off[G];  // row i of the group's list, c[j] <= i < c[j+1], is row i + off[j] of P
-      bool own[G];
+      // Few rows per latent and most latents without any: the latents come from the list that
+      // seg_class_scatter_kernel wrote, ordered by row count (those without rows first: they are
+      // zeroed by seg_zero_rows_kernel and skipped here; those with more than kSegChunk rows are not
+      // in it).  A group serves G consecutive entries, i.e. G latents of (nearly always) the same row
+      // count, so the four groups of a wavefront finish together; their rows are fetched U at a time
+      // regardless of where one latent ends and the next begins, and a latent's sum is stored when
+      // its last row has been added.  The order of the additions of a latent is the same as with G = 1.
+      // Work items: first the latents with kSegBigRows rows or more, one per group and the heaviest
+      // first (a group that had four of them would still be running long after the rest of the launch),
+      // then the others, G per group.
+      const uint32_t lo = cls_begin[1], mid = cls_begin[kSegBigRows], hi = cls_begin[kSegChunk + 1];
+      const int64_t n_big = static_cast<int64_t>(hi - mid);
+      int64_t first;  // first entry of this group
+      int count;      // entries it serves
+      if (fb < n_big) {
+        first = static_cast<int64_t>(hi) - 1 - fb;
+        count = 1;
+      } else {
+        first = static_cast<int64_t>(lo) + (fb - n_big) * G;
+        const int64_t left = static_cast<int64_t>(mid) - first;
+        count = left < G ? (left > 0 ? static_cast<int>(left) : 0) : G;
+      }
+      uint32_t fv = 0, b0v = 0, b1v = 0;  // lane j < count of the group: entry j, its latent and rows
+      if (sub < count) {
+        fv = cls_list[first + sub];
+        b0v = begin[fv];
+        b1v = begin[fv + 1];
+      }
+      uint32_t c[G + 1], off[G], fid[G];  // row i of the group's list, c[j] <= i < c[j+1], is row i + off[j] of P
       c[0] = 0;
 #pragma unroll
       for (int j = 0; j < G; ++j) {
-        const uint32_t b0 = static_cast<uint32_t>(__shfl(static_cast<int>(bv), j, kPieceLanes));
-        const uint32_t b1 = static_cast<uint32_t>(__shfl(static_cast<int>(bv), j + 1, kPieceLanes));
-        const uint32_t n = b1 - b0;
-        own[j] = f0 + j < F && n <= static_cast<uint32_t>(kSegChunk);
-        c[j + 1] = c[j] + (own[j] ? n : 0u);
+        const uint32_t b0 = static_cast<uint32_t>(__shfl(static_cast<int>(b0v), j, kPieceLanes));
+        const uint32_t b1 = static_cast<uint32_t>(__shfl(static_cast<int>(b1v), j, kPieceLanes));
+        fid[j] = static_cast<uint32_t>(__shfl(static_cast<int>(fv), j, kPieceLanes));
+        c[j + 1] = c[j] + (b1 - b0);  // nothing for entries beyond the list
         off[j] = b0 - c[j];
       }
-      float zero[EV];
-#pragma unroll
-      for (int i = 0; i < EV; ++i) zero[i] = 0.f;
-#pragma unroll
-      for (int j = 0; j < G; ++j)  // latents without rows
-        if (own[j] && c[j + 1] == c[j] && d0 < D && !update)
-          store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, (f0 + j) * D + d0, zero);
       const uint32_t total = c[G];
       for (uint32_t i0 = 0; __any(i0 < total); i0 += U) {
         raw_vec_t<PT, EV> raw[U];
-        int which[U];
+        uint32_t whose[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t i = i0 + u;
           raw[u] = raw_vec_t<PT, EV>{};
-          which[u] = 0;
+          whose[u] = fid[0];
           uint32_t o = off[0];
 #pragma unroll
           for (int j = 1; j < G; ++j)
             if (i >= c[j]) {
-              which[u] = j;
+              whose[u] = fid[j];
               o = off[j];
             }
           if (i < total)
@@ -317,7 +332,7 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
 #pragma unroll
               for (int k = 0; k < EV; ++k) acc[k] *= g;
             }
-            emit(f0 + which[u], d0, acc);
+            emit(static_cast<int64_t>(whose[u]), d0, acc);
 #pragma unroll
             for (int k = 0; k < EV; ++k) acc[k] = 0.f;
           }
@@ -450,14 +465,17 @@ __global__ void seg_find_long_kernel(const uint32_t *__restrict__ begin, int64_t
 }
 
 // chunk_begin[i] = number of chunks of the long latents before long_list[i]
-// (chunk_begin[n_long] = total); single block.
+// (chunk_begin[n_long] = total); single block.  Also clears zero_me[0..n_zero) when given (n_zero <= 1024).
 __global__ __launch_bounds__(1024) void seg_chunk_table_kernel(const uint32_t *__restrict__ begin,
                                                                const uint32_t *__restrict__ long_count,
                                                                const uint32_t *__restrict__ long_list,
-                                                               uint32_t *__restrict__ chunk_begin) {
+                                                               uint32_t *__restrict__ chunk_begin,
+                                                               uint32_t *__restrict__ zero_me, int n_zero) {
   __shared__ uint32_t wave_tot[1024 / kWave];
   __shared__ uint32_t carry_s;
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid >> 6;
+  // counters of the kernels that follow in the stream (the class histogram and cursors below)
+  if (zero_me && tid < n_zero) zero_me[tid] = 0u;
   const uint32_t n_long = *long_count;
   if (tid == 0) carry_s = 0;
   __syncthreads();
@@ -485,6 +503,99 @@ __global__ __launch_bounds__(1024) void seg_chunk_table_kernel(const uint32_t *_
     __syncthreads();
   }
   if (tid == 0) chunk_begin[n_long] = carry_s;
+}
+
+// ---- latents ordered by row count ----------------------------------------------------------
+// Where most latents have no pair at all and the rest one or a few (B*K <= 2F, skewed indices), the
+// reduction by pieces works from a list of the latents ordered by their number of rows:
+//   cls_list[cls_begin[n] .. cls_begin[n+1]) = the latents with exactly n rows, 0 <= n <= kSegChunk
+// (any order inside a class; latents with more rows are not listed: they go through the chunked
+// path).  Class 0 is zeroed in one pass over whole rows of the output (seg_zero_rows_kernel); the
+// groups of lanes of the reduction take four consecutive entries of the classes 1..kSegChunk, which
+// nearly always have the same row count, so no load slot is wasted on unequal groups.
+// Two launches: a histogram over the classes, then the placement (a counting sort whose cursors
+// are advanced once per block and class).  hist, cursor: kSegClasses counters each, zero on entry.
+constexpr int kClassPerThread = 8;  // latents per thread of the placement kernel
+
+__global__ __launch_bounds__(256) void seg_class_hist_kernel(const uint32_t *__restrict__ begin, int64_t F,
+                                                             uint32_t *__restrict__ hist) {
+  __shared__ uint32_t h[kSegClasses];
+  for (int t = threadIdx.x; t < kSegClasses; t += 256) h[t] = 0u;
+  __syncthreads();
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t f0 = static_cast<int64_t>(blockIdx.x) * blockDim.x; f0 < F; f0 += stride) {  // uniform per block
+    const int64_t f = f0 + threadIdx.x;
+    uint32_t n = kSegClasses;  // not counted
+    if (f < F) n = begin[f + 1] - begin[f];
+    // the empty class is the common one: counted per wavefront, not per lane
+    const unsigned long long empties = __ballot(n == 0u);
+    if (lane_id() == 0 && empties) atomicAdd(&h[0], static_cast<uint32_t>(__popcll(empties)));
+    if (n != 0u && n < static_cast<uint32_t>(kSegClasses)) atomicAdd(&h[n], 1u);
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < kSegClasses; t += 256)
+    if (h[t]) atomicAdd(&hist[t], h[t]);
+}
+
+__global__ __launch_bounds__(256) void seg_class_scatter_kernel(const uint32_t *__restrict__ begin, int64_t F,
+                                                                const uint32_t *__restrict__ hist,
+                                                                uint32_t *__restrict__ cursor,
+                                                                uint32_t *__restrict__ cls_begin,
+                                                                uint32_t *__restrict__ cls_list) {
+  __shared__ uint32_t base[kSegClasses + 1];  // first entry of every class
+  __shared__ uint32_t cnt[kSegClasses];       // this block's latents per class, then where they start in the class
+  const int tid = threadIdx.x;
+  if (tid <= kSegClasses) {
+    uint32_t s = 0;
+    for (int k = 0; k < tid; ++k) s += hist[k];
+    base[tid] = s;
+    if (blockIdx.x == 0) cls_begin[tid] = s;
+  }
+  if (tid < kSegClasses) cnt[tid] = 0u;
+  __syncthreads();
+  const int64_t f_block = static_cast<int64_t>(blockIdx.x) * (256 * kClassPerThread);
+  uint32_t cls[kClassPerThread], rank[kClassPerThread];
+#pragma unroll
+  for (int i = 0; i < kClassPerThread; ++i) {
+    const int64_t f = f_block + i * 256 + tid;
+    cls[i] = kSegClasses;  // not listed
+    rank[i] = 0u;
+    if (f < F) {
+      const uint32_t n = begin[f + 1] - begin[f];
+      if (n < static_cast<uint32_t>(kSegClasses)) cls[i] = n;
+    }
+    if (cls[i] < static_cast<uint32_t>(kSegClasses)) rank[i] = atomicAdd(&cnt[cls[i]], 1u);
+  }
+  __syncthreads();
+  if (tid < kSegClasses) {
+    const uint32_t c = cnt[tid];
+    cnt[tid] = c ? atomicAdd(&cursor[tid], c) : 0u;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kClassPerThread; ++i)
+    if (cls[i] < static_cast<uint32_t>(kSegClasses))
+      cls_list[base[cls[i]] + cnt[cls[i]] + rank[i]] = static_cast<uint32_t>(f_block + i * 256 + tid);
+}
+
+// out[f, 0..D) = 0 for the latents without rows (class 0 of the list): one wavefront per row, EV
+// columns per lane like the reduction by pieces (D is a multiple of EV and rows are 16-byte aligned
+// wherever that reduction runs).
+template <typename PT, typename GT>
+__global__ __launch_bounds__(256) void seg_zero_rows_kernel(const uint32_t *__restrict__ cls_begin,
+                                                            const uint32_t *__restrict__ cls_list,
+                                                            void *__restrict__ out, int D) {
+  constexpr int EV = 16 / static_cast<int>(sizeof(typename Traits<PT>::store_t));
+  const uint32_t n = cls_begin[1];
+  const int lane = lane_id();
+  float zero[EV];
+#pragma unroll
+  for (int i = 0; i < EV; ++i) zero[i] = 0.f;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < n; w += n_waves) {
+    const int64_t row = static_cast<int64_t>(cls_list[w]) * D;
+    for (int d = lane * EV; d < D; d += kWave * EV) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, row + d, zero);
+  }
 }
 
 }  // namespace flexsae
