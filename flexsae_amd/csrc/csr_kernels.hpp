@@ -437,12 +437,12 @@ __global__ void csr_inverse_kernel(const uint32_t *__restrict__ map, int64_t n_p
 // out[c] = scale * sum  with  scale = coef * (grad_out ? grad_out[0] : 1).
 constexpr int kColsumRows = 64;
 
-__global__ __launch_bounds__(256) void colsum_partial_kernel(const float *__restrict__ x, int64_t rows,
-                                                             int64_t ld, int cols,
-                                                             float *__restrict__ partial) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+// stage 1 for column c and row chunk `chunk`
+__device__ __forceinline__ void colsum_partial_one(const float *__restrict__ x, int64_t rows, int64_t ld, int cols,
+                                                   float *__restrict__ partial, int c, int64_t chunk) {
   if (c >= cols) return;
-  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * kColsumRows;
+  const int64_t r0 = chunk * kColsumRows;
+  if (r0 >= rows) return;
   const int64_t r1 = (r0 + kColsumRows) < rows ? (r0 + kColsumRows) : rows;
   float s = 0.f;
   int64_t r = r0;
@@ -454,7 +454,14 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const float *__rest
     for (int u = 0; u < 8; ++u) s += v[u];
   }
   for (; r < r1; ++r) s += x[r * ld + c];
-  partial[static_cast<int64_t>(blockIdx.y) * cols + c] = s;
+  partial[chunk * cols + c] = s;
+}
+
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const float *__restrict__ x, int64_t rows,
+                                                             int64_t ld, int cols,
+                                                             float *__restrict__ partial) {
+  colsum_partial_one(x, rows, ld, cols, partial, static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x),
+                     static_cast<int64_t>(blockIdx.y));
 }
 
 __global__ __launch_bounds__(256) void colsum_final_kernel(const float *__restrict__ partial,

@@ -460,6 +460,9 @@ inline int64_t hier_cols_used(const flexsae_shape *s, const HierBwdPlan &p, bool
 struct TrainArgs {
   const void *bias;
   const void *target;
+  float *loss;              // finished by the epilogue from the per-(tile, row) partials
+  int64_t n_loss_partials;
+  double inv_count;         // 1 / (B*K*D)
 };
 
 // largest K the training-step kernel holds in registers
@@ -686,13 +689,18 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
   if (flags & FLEXSAE_BWD_SKIP_EPILOGUE) return;
-  // dvals = its per-tile shares added in tile order
-  hipLaunchKernelGGL(hier_dvals_finalize_kernel, dim3(grid_for(s->B * s->K, 256, 8192)), dim3(256), 0, st, dv_part,
-                     static_cast<int>(d_used / (train ? train_tile_cols(s) : kWave * sweep_vec)), s->B * s->K, dvals);
-  // dbias = column sums of s_final over the rows, in a fixed order
-  hipLaunchKernelGGL(colsum_partial_kernel,
-                     dim3(static_cast<unsigned>(ceil_div(D, 256)), static_cast<unsigned>(n_chunks)), dim3(256),
-                     0, st, s_final, s->B, static_cast<int64_t>(d_pad), D, colsum_part);
+  // one launch: dvals = its per-tile shares added in tile order; stage 1 of dbias = column sums of
+  // s_final over the rows, in a fixed order; the loss of the training step from its partials
+  {
+    const unsigned n_colsum_blocks = static_cast<unsigned>(ceil_div(D, 256) * ceil_div(n_chunks, 4));
+    const unsigned n_dvals_blocks = grid_for(s->B * s->K, 1024, 2048);
+    hipLaunchKernelGGL(hier_epilogue_kernel, dim3(1 + n_colsum_blocks + n_dvals_blocks), dim3(1024), 0, st,
+                       train ? reinterpret_cast<const float *>(ws + pl.off_loss) : static_cast<const float *>(nullptr),
+                       train ? train->n_loss_partials : 0, train ? train->inv_count : 0.0,
+                       train ? train->loss : static_cast<float *>(nullptr), s_final, s->B,
+                       static_cast<int64_t>(d_pad), D, colsum_part, n_colsum_blocks, dv_part,
+                       static_cast<int>(d_used / (train ? train_tile_cols(s) : kWave * sweep_vec)), s->B * s->K, dvals);
+  }
   hipLaunchKernelGGL(colsum_final_kernel, dim3(static_cast<unsigned>(ceil_div(D, 256))), dim3(256), 0, st,
                      colsum_part, n_chunks, D, static_cast<const float *>(nullptr), 1.0f, dbias);
 }
@@ -749,7 +757,8 @@ void finish_pair_list(const flexsae_shape *s, const HierBwdPlan &pl, uint8_t *ws
                      reinterpret_cast<uint32_t *>(ws + pl.off_chunk), sparse ? cls : static_cast<uint32_t *>(nullptr),
                      2 * kClsStride);
   if (!sparse) return;
-  hipLaunchKernelGGL(seg_class_hist_kernel, dim3(grid_for(s->F, 256, 1024)), dim3(256), 0, st, begin, s->F, cls);
+  // few blocks: every block ends with one memory atomic per class it met, all on the same counters
+  hipLaunchKernelGGL(seg_class_hist_kernel, dim3(grid_for(s->F, 256, 128)), dim3(256), 0, st, begin, s->F, cls);
   hipLaunchKernelGGL(seg_class_scatter_kernel, dim3(static_cast<unsigned>(ceil_div(s->F, 256 * kClassPerThread))),
                      dim3(256), 0, st, begin, s->F, cls, cls + kClsStride, cls + 2 * kClsStride,
                      reinterpret_cast<uint32_t *>(ws + pl.off_cls_list));
@@ -1150,19 +1159,14 @@ int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void
   }
   const double count = static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D);
   const float coef = static_cast<float>(2.0 / count);
-  const TrainArgs ta = {bias, target};
+  const TrainArgs ta = {bias, target, loss, s->B * (hier_cols_used(s, pl, true, piece) / train_tile_cols(s)),
+                        1.0 / count};
   // without dW the reductions are left out like in the deferred case (dW_dtype only selects a template then)
   launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, sgd_step, coef, dW,
                           no_dw ? s->weight_dtype : dW_dtype, dvals, dbias, ws,
                           (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE)) |
                               (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0) | (sgd_step ? kBwdSgdUpdate : 0),
                           status_flag, st, &ta, piece ? static_cast<int>(piece_cols(pl)) : 0);
-  rc = launch_status();
-  if (rc != FLEXSAE_OK || (flags & FLEXSAE_BWD_SKIP_EPILOGUE)) return rc;
-  hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(1024), 0, st,
-                     reinterpret_cast<const float *>(ws + pl.off_loss),
-                     s->B * (hier_cols_used(s, pl, true, piece) / train_tile_cols(s)), 1.0 / count,
-                     loss);
   return launch_status();
 }
 

@@ -109,10 +109,9 @@ __global__ __launch_bounds__(256) void sae_fwd_kernel(
 
 // loss[0] = inv_count * sum(partial[0..n)), one block, fixed summation order, double
 // accumulation (n is B * ntiles, up to a few million).
-__global__ __launch_bounds__(1024) void loss_finalize_kernel(const float *__restrict__ partial,
-                                                             int64_t n, double inv_count,
-                                                             float *__restrict__ loss) {
-  __shared__ double red[1024];
+// (the body, for a block of 1024 threads; `red` is 1024 doubles of LDS)
+__device__ __forceinline__ void loss_finalize_block(const float *__restrict__ partial, int64_t n, double inv_count,
+                                                    float *__restrict__ loss, double *red) {
   double s = 0.0;
   int64_t i = threadIdx.x;
   for (; i + 7 * 1024 < n; i += 8 * 1024) {  // eight independent loads in flight
@@ -130,6 +129,13 @@ __global__ __launch_bounds__(1024) void loss_finalize_kernel(const float *__rest
     __syncthreads();
   }
   if (threadIdx.x == 0) loss[0] = static_cast<float>(red[0] * inv_count);
+}
+
+__global__ __launch_bounds__(1024) void loss_finalize_kernel(const float *__restrict__ partial,
+                                                             int64_t n, double inv_count,
+                                                             float *__restrict__ loss) {
+  __shared__ double red[1024];
+  loss_finalize_block(partial, n, inv_count, loss, red);
 }
 
 }  // namespace flexsae

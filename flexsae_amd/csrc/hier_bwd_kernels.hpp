@@ -2,6 +2,8 @@
 #pragma once
 
 #include "common.hpp"
+#include "csr_kernels.hpp"
+#include "fwd_kernels.hpp"
 
 namespace flexsae {
 
@@ -234,6 +236,40 @@ __global__ void hier_dvals_finalize_kernel(const float *__restrict__ dv_part, in
                                            float *__restrict__ dvals) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < n_pairs; p += stride) {
+    float acc = 0.f;
+    for (int t = 0; t < n_tiles; ++t) acc += dv_part[t * n_pairs + p];
+    dvals[p] = acc;
+  }
+}
+
+// What follows the slices of a hierarchical step, in one launch of 1024-thread blocks (the three
+// parts are independent; each computes what its own kernel computes, bit for bit):
+//   block 0                 the loss from the per-(tile, row) partials (loss_finalize_kernel), when
+//                           loss_partial is given;
+//   the next n_colsum_blocks stage 1 of the column sums of s_final (colsum_partial_kernel): a block
+//                           takes 256 columns of four consecutive row chunks;
+//   the rest                dvals from its per-tile shares (hier_dvals_finalize_kernel).
+__global__ __launch_bounds__(1024) void hier_epilogue_kernel(
+    const float *__restrict__ loss_partial, int64_t n_loss_partials, double inv_count, float *__restrict__ loss,
+    const float *__restrict__ s_final, int64_t rows, int64_t ld, int cols, float *__restrict__ colsum_part,
+    unsigned n_colsum_blocks, const float *__restrict__ dv_part, int n_tiles, int64_t n_pairs,
+    float *__restrict__ dvals) {
+  __shared__ double red[1024];
+  if (blockIdx.x == 0) {
+    if (loss_partial) loss_finalize_block(loss_partial, n_loss_partials, inv_count, loss, red);
+    return;
+  }
+  const unsigned blk = blockIdx.x - 1;
+  if (blk < n_colsum_blocks) {
+    const unsigned col_blocks = static_cast<unsigned>((cols + 255) / 256);
+    const unsigned bx = blk % col_blocks, by = blk / col_blocks;
+    colsum_partial_one(s_final, rows, ld, cols, colsum_part, static_cast<int>(bx * 256 + (threadIdx.x & 255)),
+                       static_cast<int64_t>(by) * 4 + (threadIdx.x >> 8));
+    return;
+  }
+  const int64_t n_blocks = static_cast<int64_t>(gridDim.x) - 1 - n_colsum_blocks;
+  const int64_t stride = n_blocks * 1024;
+  for (int64_t p = static_cast<int64_t>(blk - n_colsum_blocks) * 1024 + threadIdx.x; p < n_pairs; p += stride) {
     float acc = 0.f;
     for (int t = 0; t < n_tiles; ++t) acc += dv_part[t * n_pairs + p];
     dvals[p] = acc;
