@@ -190,6 +190,49 @@ def test_sgd_step_entry_point(shape, dtype):
         assert (upd - ref).abs().max() <= tol * ref.abs().max() + quant
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("D", [384, 256, 72])
+def test_sparse_latents_take_the_row_count_list(D, dtype):
+    """B*K <= 2F with skewed indices: most latents have no pair, the others between one and several
+    hundred.  The reduction then works from the list of latents ordered by row count and the rows of
+    latents without pairs are zeroed in one pass: every row of dW (handed over full of NaN) must come
+    out written, exactly zero where the latent has no pair, equal to the oracle elsewhere, for slices
+    of one, three and all column pieces; the in-place SGD variant must leave the rows without pairs
+    alone and move the others by the same gradient."""
+    B, K, F = 768, 16, 8192
+    _announce("sparse class list", (B, K, F, D), dtype)
+    args = make_inputs(B, K, F, D, dtype=dtype, seed=101, zipf_s=1.1, sort_vals=True, w_std=0.05)
+    counts = torch.bincount(args[0].flatten(), minlength=F)
+    assert B * K <= 2 * F and (counts == 0).sum() > F // 2 and counts.max() > 64
+    assert len(set(counts[(counts > 0) & (counts <= 64)].tolist())) >= 12  # many row-count classes in use
+    idx, W, v, b, t = _to_dev(args)
+    L, rW, rv, rb = oracle.loss_grads(oracle.HIER, *args, grad_out=1.0)
+    rW = torch.from_numpy(rW)
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-4
+    first = None
+    for cols in (0, 3 * 128, 1 << 20):
+        rc, loss, dW, dv, db = abi.hier_train(idx, W, v, b, t, slice_cols=cols, dw_dtype=dtype)
+        torch.cuda.synchronize()
+        assert rc == 0, _lib.status_string(rc)
+        dWc = dW.float().cpu()
+        assert not torch.isnan(dWc).any()
+        assert (dWc[counts == 0] == 0).all()
+        check_gradient("dW", dWc, rW, dtype, tol)
+        assert rel_err(dv.cpu(), rv) < tol and rel_err(db.cpu(), rb) < tol
+        if first is None:
+            first = dW
+        assert torch.equal(dW, first)  # same bits for any slice width
+    step = 0.25
+    Wn = W.clone()
+    rc, loss2, dv2, db2 = abi.hier_sgd_step(idx, Wn, v, b, t, step)
+    torch.cuda.synchronize()
+    assert rc == 0, _lib.status_string(rc)
+    assert torch.equal(Wn[(counts == 0).to(Wn.device)], W[(counts == 0).to(W.device)])
+    upd = ((W.float() - Wn.float()) / step).cpu()
+    quant = torch.finfo(dtype).eps * args[1].float().abs().max() / step
+    assert (upd - rW.float()).abs().max() <= tol * rW.abs().max() + quant
+
+
 def test_sgd_step_through_the_package():
     """hierarchical_sae_sgd_step: one fused call equals loss.backward() + plain SGD on the decoder
     weight; dvals and dbias are those of the autograd path; repeated steps lower the loss."""
