@@ -395,6 +395,19 @@ def main():
         elif rec:
             traffic_source = (f"none: profiles/hbm_traffic.json[{traffic_key}] was measured on build "
                               f"{rec.get('build_id')}, this is build {build_id}")
+    # What the memory system gives a plain kernel for the same number of bytes: the runtime's own
+    # device-to-device copy of half the launch's traffic (read once, written once).
+    moved = traffic if traffic else int(sweep_launch_bytes + B * K * slice_w * p_size)
+    copy_src = torch.empty(moved // 2, dtype=torch.uint8, device=dev)
+    copy_dst = torch.empty_like(copy_src)
+    n_copies = max(1, n_slices)  # as many back-to-back launches per timed bracket as the kernel has
+
+    def copy_launch():
+        for _ in range(n_copies):
+            copy_dst.copy_(copy_src)
+
+    copy_ms = time_kernel_events(torch, lambda: None, copy_launch, max(10, args.steps // 2), 2) / n_copies
+    del copy_src, copy_dst
     roofline = {
         "bound": "hbm",
         "kernel": sweep_name,
@@ -407,6 +420,11 @@ def main():
         "algorithmic_bytes_per_launch": int(sweep_launch_bytes),
         "avg_launch_ms": round(sweep_launch_ms, 4),
         "launches_per_step": n_slices,
+        "traffic_GBps": round(gbps(traffic, sweep_launch_ms), 1) if traffic else None,
+        "device_copy_same_bytes": {"bytes_moved": 2 * (moved // 2), "ms": round(copy_ms, 4),
+                                   "GBps": round(gbps(2 * (moved // 2), copy_ms), 1),
+                                   "what": "torch's device-to-device copy moving as many bytes as one launch of the "
+                                           "kernel (half read, half written), timed the same way"},
     }
 
     out = {
