@@ -13,6 +13,7 @@ import torch
 
 import abi
 import flexsae_amd as flex
+from flexsae_amd import _lib
 import oracle
 from helpers import DTYPE_TO_TOLS, PARAMS, REL_TOL, make_inputs, rel_err
 
