@@ -492,7 +492,7 @@ template <typename WT, typename PT, int KMAX, int VEC = 2>
 void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
                          const void *weight, const void *vals, float coef, const uint32_t *slot, void *P,
                          float *dvals, float *s_final, int d_pad, float *loss_partial, int *status_flag,
-                         int64_t cols, int col0, int slice_w, hipStream_t st) {
+                         int64_t cols, int col0, int slice_w, hipStream_t st, const HotFinalize &fin) {
   constexpr int LDSROWS = train_lds_rows<WT, KMAX, VEC>();
   const int64_t n_items = s->B * (cols / (kWave * VEC));
   // K == KMAX (the usual powers of two) runs the variant without per-step bound tests, part of its
@@ -503,20 +503,21 @@ void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int6
                                     : hier_train_kernel<WT, PT, KMAX, true, false, VEC, LDSROWS>)
                           : (stream ? hier_train_kernel<WT, PT, KMAX, false, true, VEC, 0>
                                     : hier_train_kernel<WT, PT, KMAX, false, false, VEC, 0>);
-  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock), 0, st,
-                     indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
+  hipLaunchKernelGGL(kernel, dim3(fin.n_blocks + static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock),
+                     0, st, indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
                      coef, slot, P, dvals, s_final, d_pad, loss_partial, status_flag, n_items, s->B, col0,
-                     slice_w, static_cast<int>(s->K), s->F, static_cast<int>(s->D));
+                     slice_w, static_cast<int>(s->K), s->F, static_cast<int>(s->D), fin);
 }
 
 template <typename WT, typename PT>
 void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
                            const void *weight, const void *vals, float coef, const uint32_t *slot, void *P,
                            float *dvals, float *s_final, int d_pad, float *loss_partial,
-                           int *status_flag, int64_t cols, int col0, int slice_w, hipStream_t st) {
+                           int *status_flag, int64_t cols, int col0, int slice_w, hipStream_t st,
+                           const HotFinalize &fin) {
 #define FLEXSAE_TRAIN(KM)                                                                              \
   launch_train_kernel<WT, PT, KM>(s, ta, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,  \
-                                  loss_partial, status_flag, cols, col0, slice_w, st)
+                                  loss_partial, status_flag, cols, col0, slice_w, st, fin)
   // (the fp32 16-step instantiation allocates registers badly; 32 covers it)
   if (s->K <= 16 && sizeof(typename Traits<WT>::store_t) == 2) {
     FLEXSAE_TRAIN(16);
@@ -532,10 +533,10 @@ void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const in
     }
   } else if (s->K <= 128) {  // fp32 rows of 65..128 steps: one column per lane
     launch_train_kernel<WT, PT, 128, 1>(s, ta, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,
-                                        loss_partial, status_flag, cols, col0, slice_w, st);
+                                        loss_partial, status_flag, cols, col0, slice_w, st, fin);
   } else {
     launch_train_kernel<WT, PT, 256, 1>(s, ta, indices, weight, vals, coef, slot, P, dvals, s_final, d_pad,
-                                        loss_partial, status_flag, cols, col0, slice_w, st);
+                                        loss_partial, status_flag, cols, col0, slice_w, st, fin);
   }
 #undef FLEXSAE_TRAIN
 }
@@ -558,7 +559,19 @@ template <typename PT, typename GT, int VEC>
 void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc, const uint32_t *chunk_begin,
                        const void *P, float *partial, void *dW, const float *dw_scale, int64_t F, int tps,
                        int col0, int sw, int D, hipStream_t st, int piece_cols = 0, int64_t cols = 0, int64_t n_pairs = 0,
-                       int update = 0, const uint32_t *cls_begin = nullptr, const uint32_t *cls_list = nullptr) {
+                       int update = 0, const uint32_t *cls_begin = nullptr, const uint32_t *cls_list = nullptr,
+                       HotFinalize *defer = nullptr) {
+  // the second step of the hot latents: launched here, or handed back through `defer` for the next
+  // training-step launch to carry
+  auto finalize = [&](int mode, int units) {
+    HotFinalize h = {sc.long_count, sc.long_list, chunk_begin, partial, dW, dw_scale, mode, units, col0, sw, D, update, 256u};
+    if (defer) {
+      h.n_blocks = 64u;  // riding along with a long launch: few blocks, so that they cost little where there is nothing to do
+      *defer = h;
+    }
+    else
+      hipLaunchKernelGGL((hot_finalize_kernel<GT>), dim3(h.n_blocks), dim3(kBlock), 0, st, h);
+  };
   if (piece_cols > 0) {  // 256-byte pieces, sixteen lanes each
     const int pps = static_cast<int>(cols / piece_cols);
     int pps_shift = -1;  // log2(pps) when pps is a power of two
@@ -583,9 +596,7 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
     }
 #undef FLEXSAE_PIECE_REDUCE
     // the chunk partials of hot latents are combined per 64-column piece
-    hipLaunchKernelGGL((seg_reduce_piece_finalize_kernel<GT>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
-                       sc.long_list, chunk_begin, partial, dW, dw_scale, static_cast<int>(cols / kWave), col0, sw, D,
-                       update);
+    finalize(1, static_cast<int>(cols / kWave));
     return;
   }
   constexpr bool kCanNarrow = sizeof(typename Traits<PT>::store_t) == 4 && VEC == 4;
@@ -596,16 +607,20 @@ void launch_seg_reduce(bool narrow, const uint32_t *begin, const CsrScratch &sc,
     hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, RV, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks),
                        dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale,
                        F, kLongBlocks, rtps, col0, sw, D);
-    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, RV, 8>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
-                       sc.long_list, chunk_begin, partial, dW, dw_scale, rtps, col0, sw, D);
+    static_assert(RV == 2 || !kCanNarrow, "the narrow reduction works on tiles of 128 columns");
+    finalize(3, rtps);
     return;
   }
   const unsigned n_short_blocks = static_cast<unsigned>(ceil_div(F * tps, kWavesPerBlock));
   hipLaunchKernelGGL((seg_reduce_kernel<PT, GT, VEC, FLEXSAE_REDUCE_U>), dim3(kLongBlocks + n_short_blocks),
                      dim3(kBlock), 0, st, begin, sc.long_count, sc.long_list, chunk_begin, P, partial, dW, dw_scale, F,
                      kLongBlocks, tps, col0, sw, D);
-  hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
-                     sc.long_list, chunk_begin, partial, dW, dw_scale, tps, col0, sw, D);
+  if constexpr (VEC == 4) {
+    finalize(2, tps);
+  } else {
+    hipLaunchKernelGGL((seg_reduce_long_finalize_kernel<GT, VEC, 8>), dim3(256), dim3(kBlock), 0, st, sc.long_count,
+                       sc.long_list, chunk_begin, partial, dW, dw_scale, tps, col0, sw, D);
+  }
 }
 
 template <typename WT, typename PT, typename GT, int VEC>
@@ -650,13 +665,19 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const uint32_t *cls_list = reinterpret_cast<const uint32_t *>(ws + pl.off_cls_list);
   if (sparse && do_reduce && !update)
     hipLaunchKernelGGL((seg_zero_rows_kernel<PT, GT>), dim3(2048), dim3(kBlock), 0, st, cls_begin, cls_list, dW, D);
+  // In the training step the second step of a slice's hot latents travels with the next slice's
+  // training-step launch (a gradient of the weight's own dtype only: that is what that kernel writes);
+  // the last slice's gets a launch of its own.
+  HotFinalize pending = {};
+  const bool fold = std::is_same<GT, WT>::value && train != nullptr && do_sweep && do_reduce;
   for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (d_used - col0) < slice_w ? (d_used - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
     if (train && do_sweep) {
       launch_train_kernel_k<WT, PT>(s, *train, indices, weight, vals, coef, slot, P, dv_part, s_final, d_pad,
                                     reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
-                                    static_cast<int>(col0), sw, st);
+                                    static_cast<int>(col0), sw, st, pending);
+      pending = HotFinalize{};
     } else if (do_sweep) {
 #define FLEXSAE_SWEEP(SV)                                                                                      \
   hipLaunchKernelGGL((hier_sweep_kernel<WT, PT, SV, FLEXSAE_SWEEP_U>),                                         \
@@ -684,7 +705,11 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
         piece != 0 && (update || cols % pl.tile != 0 || s->B * s->K <= 2 * s->F || cache_sized);
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
                                    static_cast<int>(col0), sw, D, st, by_pieces ? piece : 0, cols, s->B * s->K, update,
-                                   sparse ? cls_begin : nullptr, sparse ? cls_list : nullptr);
+                                   sparse ? cls_begin : nullptr, sparse ? cls_list : nullptr, fold ? &pending : nullptr);
+  }
+  if (pending.n_blocks != 0) {
+    pending.n_blocks = 256u;
+    hipLaunchKernelGGL((hot_finalize_kernel<GT>), dim3(pending.n_blocks), dim3(kBlock), 0, st, pending);
   }
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only

@@ -2,6 +2,7 @@
 #pragma once
 
 #include "common.hpp"
+#include "segment_kernels.hpp"
 
 namespace flexsae {
 
@@ -67,6 +68,8 @@ struct RowPiece<f16_t, 2> {
 // back with plain LDS loads.  bias - target is fetched before the gathers are issued: the memory
 // counter retires in order, so anything issued after them can only be waited for together with
 // all of them, and the forward walk could not start while rows are still arriving.
+// fin: the second step of the previous slice's hot latents (see HotFinalize), run by the leading blocks
+// of the launch into a gradient of the weight's own dtype.
 // STREAM: the contributions are stored with the non-temporal hint.  That is the faster choice
 // when all of P is written before any of it is read back (it is far larger than the caches);
 // when P is one slice that the reduction reads right after this launch, plain stores leave part
@@ -78,7 +81,7 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     const void *__restrict__ target, int target_dtype, float coef,
     const uint32_t *__restrict__ slot, void *__restrict__ P, float *__restrict__ dv_part,
     float *__restrict__ s_final, int s_final_ld, float *__restrict__ loss_partial,
-    int *status_flag, int64_t n_items, int64_t B, int col0, int slice_w, int K, int64_t F, int D) {
+    int *status_flag, int64_t n_items, int64_t B, int col0, int slice_w, int K, int64_t F, int D, HotFinalize fin) {
   using Piece = RowPiece<WT, VEC>;
   using raw_t = typename Piece::raw_t;
   using S_t = typename Traits<WT>::store_t;
@@ -89,7 +92,12 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   __shared__ uint32_t lds_rows[LDSROWS > 0 ? (256 / kWave) * LDSROWS * kWave : 1];
   uint32_t *const my_lds = lds_rows + wave_in_block() * (LDSROWS * kWave);
   const int lane = lane_id();
-  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+  // the leading blocks finish the hot latents of the previous slice (fin.n_blocks of them; none at the first slice)
+  if (blockIdx.x < fin.n_blocks) {
+    hot_finalize_run<WT>(fin, blockIdx.x);
+    return;
+  }
+  const int64_t item = static_cast<int64_t>(blockIdx.x - fin.n_blocks) * (blockDim.x >> 6) + wave_in_block();
   if (item >= n_items) return;  // uniform per wavefront
   const int t = static_cast<int>(item / B);
   const int64_t b = item - static_cast<int64_t>(t) * B;

@@ -366,22 +366,24 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_kernel(
   }
 }
 
-// Long latents of the piece reduction, second launch: out[f, slice] = sum of the latent's chunk
+// Long latents of the piece reduction, second step: out[f, slice] = sum of the latent's chunk
 // partials in a fixed order.  One wavefront per (long latent, 64-column piece of the fp32
-// partials); its four groups take every fourth chunk and are added up as above.
+// partials); its four groups take every fourth chunk and are added up as above.  `block` of
+// `n_blocks` blocks of 256 threads share the work (a launch of its own, or the leading blocks of
+// the next slice's training-step launch).
 template <typename GT>
-__global__ __launch_bounds__(256) void seg_reduce_piece_finalize_kernel(
+__device__ __forceinline__ void seg_piece_finalize_body(
     const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
     const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
     void *__restrict__ out, const float *__restrict__ scale, int pieces, int col0, int slice_w, int D,
-    int update) {
+    int update, unsigned block, unsigned n_blocks) {
   constexpr int EV = 4, U = 4, kGroups = kWave / kPieceLanes;
   const int lane = lane_id();
   const int sub = lane & (kPieceLanes - 1), g = lane / kPieceLanes;
   const uint32_t n_long = *long_count;
   const int64_t total = static_cast<int64_t>(n_long) * pieces;
-  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
-  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total; w += n_waves) {
+  const int64_t n_waves = static_cast<int64_t>(n_blocks) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(block) * (blockDim.x >> 6) + wave_in_block(); w < total; w += n_waves) {
     const uint32_t i = static_cast<uint32_t>(w / pieces);
     const int t = static_cast<int>(w - static_cast<int64_t>(i) * pieces);
     const int pc = t * (kPieceLanes * EV) + sub * EV;
@@ -423,17 +425,29 @@ __global__ __launch_bounds__(256) void seg_reduce_piece_finalize_kernel(
   }
 }
 
-// Long latents, second launch: out[f, slice] = sum of the latent's chunk partials, in chunk order.
-template <typename GT, int VEC, int U>
-__global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
+template <typename GT>
+__global__ __launch_bounds__(256) void seg_reduce_piece_finalize_kernel(
     const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
     const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
-    void *__restrict__ out, const float *__restrict__ scale, int tps, int col0, int slice_w, int D) {
+    void *__restrict__ out, const float *__restrict__ scale, int pieces, int col0, int slice_w, int D,
+    int update) {
+  seg_piece_finalize_body<GT>(long_count, long_list, chunk_begin, partial, out, scale, pieces, col0, slice_w, D, update,
+                              blockIdx.x, gridDim.x);
+}
+
+// Long latents, second step of the reduction by tiles: out[f, slice] = sum of the latent's chunk
+// partials, in chunk order.
+template <typename GT, int VEC, int U>
+__device__ __forceinline__ void seg_long_finalize_body(
+    const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
+    const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
+    void *__restrict__ out, const float *__restrict__ scale, int tps, int col0, int slice_w, int D,
+    unsigned block, unsigned n_blocks) {
   const int lane = lane_id();
   const uint32_t n_long = *long_count;
   const int64_t total = static_cast<int64_t>(n_long) * tps;
-  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
-  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < total;
+  const int64_t n_waves = static_cast<int64_t>(n_blocks) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(block) * (blockDim.x >> 6) + wave_in_block(); w < total;
        w += n_waves) {
     const uint32_t i = static_cast<uint32_t>(w / tps);
     const int t = static_cast<int>(w - static_cast<int64_t>(i) * tps);
@@ -451,6 +465,50 @@ __global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
     }
     if (d0 < D) store_vec<GT, VEC>(out, static_cast<int64_t>(long_list[i]) * D + d0, acc);
   }
+}
+
+template <typename GT, int VEC, int U>
+__global__ __launch_bounds__(256) void seg_reduce_long_finalize_kernel(
+    const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ long_list,
+    const uint32_t *__restrict__ chunk_begin, const float *__restrict__ partial,
+    void *__restrict__ out, const float *__restrict__ scale, int tps, int col0, int slice_w, int D) {
+  seg_long_finalize_body<GT, VEC, U>(long_count, long_list, chunk_begin, partial, out, scale, tps, col0, slice_w, D,
+                                     blockIdx.x, gridDim.x);
+}
+
+// The second step of a slice's hot latents as a parcel that another launch can carry: the
+// training-step kernel of the next slice runs it in its leading blocks (it touches neither the
+// contributions nor the partial sums, and the reduction that overwrites the partial sums comes after
+// it in the stream), which saves a launch per slice.
+struct HotFinalize {
+  const uint32_t *long_count;
+  const uint32_t *long_list;
+  const uint32_t *chunk_begin;
+  const float *partial;
+  void *out;
+  const float *scale;
+  int mode;   // 0: nothing, 1: pieces of 64 columns, 2: tiles of 256 columns, 3: tiles of 128 columns
+  int units;  // pieces or tiles per slice
+  int col0, slice_w, D, update;
+  unsigned n_blocks;  // blocks of 256 threads that share it
+};
+
+template <typename GT>
+__device__ __forceinline__ void hot_finalize_run(const HotFinalize &h, unsigned block) {
+  if (h.mode == 1)
+    seg_piece_finalize_body<GT>(h.long_count, h.long_list, h.chunk_begin, h.partial, h.out, h.scale, h.units, h.col0,
+                                h.slice_w, h.D, h.update, block, h.n_blocks);
+  else if (h.mode == 2)
+    seg_long_finalize_body<GT, 4, 8>(h.long_count, h.long_list, h.chunk_begin, h.partial, h.out, h.scale, h.units,
+                                     h.col0, h.slice_w, h.D, block, h.n_blocks);
+  else if (h.mode == 3)
+    seg_long_finalize_body<GT, 2, 8>(h.long_count, h.long_list, h.chunk_begin, h.partial, h.out, h.scale, h.units,
+                                     h.col0, h.slice_w, h.D, block, h.n_blocks);
+}
+
+template <typename GT>
+__global__ __launch_bounds__(256) void hot_finalize_kernel(HotFinalize h) {
+  hot_finalize_run<GT>(h, blockIdx.x);
 }
 
 // long_list[0..*long_count) = latents with more than kSegChunk pairs (any order);
