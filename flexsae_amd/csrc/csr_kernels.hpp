@@ -196,31 +196,99 @@ __device__ __forceinline__ void block_bitonic_sort(Ptr a, uint32_t n) {
 // Long groups (more than 64 pairs): one block per group, striding over the list.  Groups of up
 // to kSortLdsElems pairs are sorted in LDS, longer ones in place in global memory.  With `slot`
 // given, the positions of the group's pairs are written there as well.
+// A latent that is in a large share of the rows (thousands of pairs) is not compared at all: a
+// pair id is row * K + step, so counting the group's pairs per row and scanning the counts places
+// every pair (a counting sort over the rows, O(pairs + rows) instead of the network's
+// O(pairs log^2 pairs)); pairs of the same row, if a row holds the latent more than once, are
+// ranked among themselves afterwards.  Taken when the rows fit the LDS counters and the network
+// would cost several times more.
 constexpr uint32_t kSortLdsElems = 8192;
+constexpr uint32_t kSortRowsMax = 8192;  // rows (B) the counting sort has LDS counters for
 __global__ __launch_bounds__(1024) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
                                                             uint32_t *__restrict__ map,
                                                             const uint32_t *__restrict__ long_count,
                                                             const uint32_t *__restrict__ long_list,
-                                                            uint32_t *__restrict__ slot) {
-  __shared__ uint32_t buf[kSortLdsElems];
+                                                            uint32_t *__restrict__ slot, uint32_t n_rows,
+                                                            uint32_t K) {
+  __shared__ uint32_t buf[kSortLdsElems];  // the group (network), or its pairs grouped by row (counting sort)
+  __shared__ uint32_t rowcnt[kSortRowsMax];
+  __shared__ uint32_t wave_tot[1024 / kWave];
   const uint32_t n_long = *long_count;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid >> 6;
   for (uint32_t w = blockIdx.x; w < n_long; w += gridDim.x) {
     const uint32_t f = long_list[w];
-    uint32_t *a = map + begin[f];
-    const uint32_t n = begin[f + 1] - begin[f];
+    const uint32_t base = begin[f];
+    uint32_t *a = map + base;
+    const uint32_t n = begin[f + 1] - base;
     if (n <= kSortLdsElems) {
-      for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) buf[i] = a[i];
+      uint32_t lg = 1;
+      while ((1u << lg) < n) ++lg;
+      // network: about n/2 * lg*(lg+1)/2 comparators; counting: a few passes over n pairs and n_rows counters
+      const bool by_rows = n_rows <= kSortRowsMax && K > 0 &&
+                           static_cast<uint64_t>(n) * lg * (lg + 1) > 4ull * (static_cast<uint64_t>(n) + n_rows);
+      if (by_rows) {  // uniform over the block
+        for (uint32_t r = tid; r < n_rows; r += blockDim.x) rowcnt[r] = 0u;
+        __syncthreads();
+        for (uint32_t i = tid; i < n; i += blockDim.x) atomicAdd(&rowcnt[a[i] / K], 1u);
+        __syncthreads();
+        // exclusive scan of rowcnt[0..n_rows): every thread owns eight consecutive counters
+        {
+          constexpr uint32_t PER = kSortRowsMax / 1024;
+          uint32_t x[PER], tsum = 0;
+#pragma unroll
+          for (uint32_t i = 0; i < PER; ++i) {
+            const uint32_t r = static_cast<uint32_t>(tid) * PER + i;
+            x[i] = r < n_rows ? rowcnt[r] : 0u;
+            tsum += x[i];
+          }
+          uint32_t inc = tsum;
+#pragma unroll
+          for (int off = 1; off < kWave; off <<= 1) {
+            const uint32_t y = __shfl_up(inc, off, kWave);
+            if (lane >= off) inc += y;
+          }
+          if (lane == kWave - 1) wave_tot[wv] = inc;
+          __syncthreads();
+          uint32_t run = inc - tsum;
+          for (int q = 0; q < wv; ++q) run += wave_tot[q];
+#pragma unroll
+          for (uint32_t i = 0; i < PER; ++i) {
+            const uint32_t r = static_cast<uint32_t>(tid) * PER + i;
+            if (r < n_rows) rowcnt[r] = run;
+            run += x[i];
+          }
+          __syncthreads();
+        }
+        // placement by row; the atomics leave rowcnt[r] at the end of row r's pairs
+        for (uint32_t i = tid; i < n; i += blockDim.x) {
+          const uint32_t id = a[i];
+          buf[atomicAdd(&rowcnt[id / K], 1u)] = id;
+        }
+        __syncthreads();
+        // pairs of one row are in the order of the atomics: rank them among themselves on the way out
+        for (uint32_t i = tid; i < n; i += blockDim.x) {
+          const uint32_t id = buf[i], r = id / K;
+          const uint32_t s0 = r ? rowcnt[r - 1] : 0u, s1 = rowcnt[r];
+          uint32_t rank = 0;
+          for (uint32_t j = s0; j < s1; ++j) rank += (buf[j] < id) ? 1u : 0u;
+          a[s0 + rank] = id;
+          if (slot) slot[id] = base + s0 + rank;
+        }
+        __syncthreads();
+        continue;
+      }
+      for (uint32_t i = tid; i < n; i += blockDim.x) buf[i] = a[i];
       __syncthreads();
       block_bitonic_sort(buf, n);
-      for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+      for (uint32_t i = tid; i < n; i += blockDim.x) {
         a[i] = buf[i];
-        if (slot) slot[buf[i]] = begin[f] + i;
+        if (slot) slot[buf[i]] = base + i;
       }
       __syncthreads();
     } else {
       block_bitonic_sort(a, n);  // ends with a barrier
       if (slot)
-        for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) slot[a[i]] = begin[f] + i;
+        for (uint32_t i = tid; i < n; i += blockDim.x) slot[a[i]] = base + i;
     }
   }
 }

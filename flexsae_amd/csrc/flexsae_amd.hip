@@ -340,8 +340,9 @@ void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
                        n_pairs, F, pl.shift, pl.n_buckets, pl.chunk, pl.n_chunks, sc.table, sc.tmp);
     hipLaunchKernelGGL(csr_bucket_sort_kernel, dim3(pl.n_buckets), dim3(kSortThreads), 0, st, sc.tmp, sc.table,
                        pl.n_chunks, pl.shift, F, begin, map, slot, sc.long_count, sc.long_list);
-    hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(1024), 0, st, begin, map, sc.long_count,
-                       sc.long_list, slot);
+    hipLaunchKernelGGL(csr_sort_long_kernel, dim3(1024), dim3(1024), 0, st, begin, map, sc.long_count,
+                       sc.long_list, slot, static_cast<uint32_t>(B < (1LL << 31) ? B : 0xffffffffLL),
+                       static_cast<uint32_t>(K));
     return;
   }
   hipLaunchKernelGGL(csr_init_kernel, dim3(grid_for(F + 1, 256, 4096)), dim3(256), 0, st, begin, F + 1,
@@ -358,8 +359,9 @@ void csr_build_launch(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
   hipLaunchKernelGGL(csr_sort_short_kernel,
                      dim3(static_cast<unsigned>(ceil_div(F, kWavesPerBlock))), dim3(kBlock), 0, st,
                      begin, map, F, sc.long_count, sc.long_list);
-  hipLaunchKernelGGL(csr_sort_long_kernel, dim3(512), dim3(1024), 0, st, begin, map, sc.long_count,
-                     sc.long_list, static_cast<uint32_t *>(nullptr));
+  hipLaunchKernelGGL(csr_sort_long_kernel, dim3(1024), dim3(1024), 0, st, begin, map, sc.long_count,
+                     sc.long_list, static_cast<uint32_t *>(nullptr), static_cast<uint32_t>(B < (1LL << 31) ? B : 0xffffffffLL),
+                     static_cast<uint32_t>(K));
   if (slot)
     hipLaunchKernelGGL(csr_inverse_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, map, n_pairs,
                        slot);
