@@ -505,8 +505,7 @@ void launch_train_kernel(const flexsae_shape *s, const TrainArgs &ta, const int6
                                     : hier_train_kernel<WT, PT, KMAX, true, false, VEC, LDSROWS>)
                           : (stream ? hier_train_kernel<WT, PT, KMAX, false, true, VEC, 0>
                                     : hier_train_kernel<WT, PT, KMAX, false, false, VEC, 0>);
-  hipLaunchKernelGGL(kernel, dim3(fin.n_blocks + fin.z_blocks + static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))),
-                     dim3(kBlock),
+  hipLaunchKernelGGL(kernel, dim3(fin.n_blocks + static_cast<unsigned>(ceil_div(n_items, kWavesPerBlock))), dim3(kBlock),
                      0, st, indices, weight, vals, s->vals_dtype, ta.bias, s->bias_dtype, ta.target, s->target_dtype,
                      coef, slot, P, dvals, s_final, d_pad, loss_partial, status_flag, n_items, s->B, col0,
                      slice_w, static_cast<int>(s->K), s->F, static_cast<int>(s->D), fin);
@@ -666,29 +665,17 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const bool sparse = piece != 0 && sparse_latents(s);
   const uint32_t *cls_begin = reinterpret_cast<const uint32_t *>(ws + pl.off_cls) + 2 * kClsStride;
   const uint32_t *cls_list = reinterpret_cast<const uint32_t *>(ws + pl.off_cls_list);
-  // (as a launch of its own, or, in the training step, shared out over the training-step launches)
-  HotFinalize pending = {};
-  const bool fold = std::is_same<GT, WT>::value && train != nullptr && do_sweep && do_reduce;
-  const int n_slices = static_cast<int>(ceil_div(s->D, slice_w));
-  const bool carry_zero = sparse && do_reduce && !update && fold;
-  if (sparse && do_reduce && !update && !carry_zero)
+  if (sparse && do_reduce && !update)
     hipLaunchKernelGGL((seg_zero_rows_kernel<PT, GT>), dim3(2048), dim3(kBlock), 0, st, cls_begin, cls_list, dW, D);
-  int slice_no = 0;
   // In the training step the second step of a slice's hot latents travels with the next slice's
   // training-step launch (a gradient of the weight's own dtype only: that is what that kernel writes);
   // the last slice's gets a launch of its own.
-  for (int64_t col0 = 0; col0 < s->D; col0 += slice_w, ++slice_no) {
+  HotFinalize pending = {};
+  const bool fold = std::is_same<GT, WT>::value && train != nullptr && do_sweep && do_reduce;
+  for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
     const int64_t cols = (d_used - col0) < slice_w ? (d_used - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
     if (train && do_sweep) {
-      if (carry_zero) {
-        pending.z_begin = cls_begin;
-        pending.z_list = cls_list;
-        pending.z_out = dW;
-        pending.z_part = slice_no;
-        pending.z_parts = n_slices;
-        pending.z_blocks = 512u;
-      }
       launch_train_kernel_k<WT, PT>(s, *train, indices, weight, vals, coef, slot, P, dv_part, s_final, d_pad,
                                     reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
                                     static_cast<int>(col0), sw, st, pending);

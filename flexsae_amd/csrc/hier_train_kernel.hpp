@@ -97,13 +97,7 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     hot_finalize_run<WT>(fin, blockIdx.x);
     return;
   }
-  if (blockIdx.x < fin.n_blocks + fin.z_blocks) {  // this launch's share of the zero pass of sparse shapes
-    seg_zero_rows_body<WT, (16 / static_cast<int>(sizeof(typename Traits<PT>::store_t)))>(fin.z_begin, fin.z_list, fin.z_out, D, blockIdx.x - fin.n_blocks,
-                                                fin.z_blocks, fin.z_part, fin.z_parts);
-    return;
-  }
-  const int64_t item =
-      static_cast<int64_t>(blockIdx.x - fin.n_blocks - fin.z_blocks) * (blockDim.x >> 6) + wave_in_block();
+  const int64_t item = static_cast<int64_t>(blockIdx.x - fin.n_blocks) * (blockDim.x >> 6) + wave_in_block();
   if (item >= n_items) return;  // uniform per wavefront
   const int t = static_cast<int>(item / B);
   const int64_t b = item - static_cast<int64_t>(t) * B;

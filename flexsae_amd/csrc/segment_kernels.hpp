@@ -491,35 +491,7 @@ struct HotFinalize {
   int units;  // pieces or tiles per slice
   int col0, slice_w, D, update;
   unsigned n_blocks;  // blocks of 256 threads that share it
-  // a share of the zero pass of sparse shapes (rows of latents without pairs), carried the same way:
-  // part z_part of z_parts of the list's class 0, by the z_blocks blocks that follow the n_blocks above
-  const uint32_t *z_begin;
-  const uint32_t *z_list;
-  void *z_out;
-  int z_part, z_parts;
-  unsigned z_blocks;
 };
-
-// out[f, 0..D) = 0 for the latents of class 0 of the row-count list (those without rows), or for share
-// `part` of `parts` of them: one wavefront per row, EV columns per lane.
-template <typename GT, int EV>
-__device__ __forceinline__ void seg_zero_rows_body(const uint32_t *__restrict__ cls_begin,
-                                                   const uint32_t *__restrict__ cls_list, void *__restrict__ out,
-                                                   int D, unsigned block, unsigned n_blocks, int part, int parts) {
-  const uint32_t n_all = cls_begin[1];
-  const uint32_t per = (n_all + static_cast<uint32_t>(parts) - 1) / static_cast<uint32_t>(parts);
-  const uint32_t lo = per * static_cast<uint32_t>(part);
-  const uint32_t hi = lo + per < n_all ? lo + per : n_all;
-  const int lane = lane_id();
-  float zero[EV];
-#pragma unroll
-  for (int i = 0; i < EV; ++i) zero[i] = 0.f;
-  const int64_t n_waves = static_cast<int64_t>(n_blocks) * (blockDim.x >> 6);
-  for (int64_t w = lo + static_cast<int64_t>(block) * (blockDim.x >> 6) + wave_in_block(); w < hi; w += n_waves) {
-    const int64_t row = static_cast<int64_t>(cls_list[w]) * D;
-    for (int d = lane * EV; d < D; d += kWave * EV) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, row + d, zero);
-  }
-}
 
 template <typename GT>
 __device__ __forceinline__ void hot_finalize_run(const HotFinalize &h, unsigned block) {
@@ -671,7 +643,17 @@ template <typename PT, typename GT>
 __global__ __launch_bounds__(256) void seg_zero_rows_kernel(const uint32_t *__restrict__ cls_begin,
                                                             const uint32_t *__restrict__ cls_list,
                                                             void *__restrict__ out, int D) {
-  seg_zero_rows_body<GT, (16 / static_cast<int>(sizeof(typename Traits<PT>::store_t)))>(cls_begin, cls_list, out, D, blockIdx.x, gridDim.x, 0, 1);
+  constexpr int EV = 16 / static_cast<int>(sizeof(typename Traits<PT>::store_t));
+  const uint32_t n = cls_begin[1];
+  const int lane = lane_id();
+  float zero[EV];
+#pragma unroll
+  for (int i = 0; i < EV; ++i) zero[i] = 0.f;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+  for (int64_t w = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(); w < n; w += n_waves) {
+    const int64_t row = static_cast<int64_t>(cls_list[w]) * D;
+    for (int d = lane * EV; d < D; d += kWave * EV) store_vec<GT, EV, FLEXSAE_REDUCE_NT>(out, row + d, zero);
+  }
 }
 
 }  // namespace flexsae
