@@ -306,7 +306,7 @@ __global__ __launch_bounds__(1024) void csr_sort_long_kernel(const uint32_t *__r
 // ---------------------------------------------------------------------------------
 constexpr int kBucketThreads = 256;
 constexpr int kBucketMaxBuckets = 8192;  // LDS counters of the count / scatter kernels
-constexpr int kSortThreads = 512;
+constexpr int kSortThreads = 1024;
 constexpr int kSortMaxLatents = 4096;    // latents per bucket (2^shift) at most
 constexpr int kSortCap = 8192;           // pairs of a bucket that are sorted inside the LDS
 
