@@ -21,6 +21,11 @@ import sys
 import time
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+# what the "algorithmic_frac_of_peak" figures of whole steps and of the forward kernel are
+ALGORITHMIC_NOTE = ("algorithmic bytes / time / 8 TB/s: every gathered row counted once per sweep whether HBM or a "
+                    "cache served it, so this is not an HBM utilisation and exceeds 1 where hot rows come from the "
+                    "L2 (skewed indices) or the weights fit the memory-side cache; roofline.traffic holds the "
+                    "counter-measured bytes of the dominant kernel")
 
 WORKLOADS = {
     # name: (B, K, F, D, dtype, index distribution, weight std)
@@ -41,6 +46,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_k128", choices=sorted(WORKLOADS))
     ap.add_argument("--shape", default="", help="override B,K,F,D of the workload (tuning aid)")
+    ap.add_argument("--dtype", default="", choices=["", "bf16", "fp16", "fp32"],
+                    help="override the storage dtype of the workload (tuning aid)")
     ap.add_argument("--no-other-mode", action="store_true",
                     help="skip the extra timing of the hierarchical loss in its other memory mode (staged / flat)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -222,8 +229,10 @@ def main():
     B, K, F, D, dt_name, dist, w_std = WORKLOADS[args.workload]
     if args.shape:
         B, K, F, D = (int(x) for x in args.shape.split(","))
-    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[dt_name]
-    es = 2 if dtype == torch.bfloat16 else 4
+    if args.dtype:
+        dt_name = args.dtype
+    dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[dt_name]
+    es = 4 if dtype == torch.float32 else 2
     inputs, generated_with = make_inputs(torch, B, K, F, D, dtype, dist, w_std, dev)
     idx, W, v, b, t = inputs
     torch.cuda.synchronize()
@@ -288,7 +297,7 @@ def main():
     dbias = torch.empty(D, dtype=torch.float32, device=dev)
     dW = torch.empty(F, D, dtype=dtype, device=dev)
     p_size = 2 if dtype == torch.bfloat16 else 4
-    scratch = flex.ops._hier_scratch_budget(K)  # FLEXSAE_HIER_SCRATCH_MB, else the package's default rule
+    scratch = flex.ops._hier_scratch_budget(B, K, F, D, dtype)  # FLEXSAE_HIER_SCRATCH_MB, else the package's rule
     # same decision as the API: the fused training step runs when the stage budget holds every
     # per-pair contribution at once (one slice as wide as D); otherwise forward + sliced backward
     # (staged); failing that, the same kernel slice by slice with an immediate reduction (sliced);
@@ -298,12 +307,17 @@ def main():
              and bool(lib.flexsae_hier_fwd_bwd_supported(ctypes.byref(sh))))
     staged = fused and flex.ops._stage_fits(idx, W)
     hier_mode = "staged" if staged else "sliced" if fused else "unfused"
-    slice_cols = D if staged else flex.ops._hier_slice_cols(B, K, p_size)
+    slice_cols = D if staged else flex.ops._hier_slice_cols(B, K, F, D, dtype)
+    # hot-latent accumulators: the same decision as the API takes for a weight that needs its gradient
+    hot = bool(fused and not staged and flex.ops._use_hot_latents(B, K, F, D, dtype))
+    HOTF = _lib.BWD_HOT_LATENTS if hot else 0
+    if hot:
+        slice_cols = flex.ops._hot_slice_cols(B, slice_cols, dev)
     tile = 64 * (4 if D % 4 == 0 else 2 if D % 2 == 0 else 1)
     d_pad = -(-D // tile) * tile
     if fused:
         # slices are whole training tiles when the reduction can work on 256-byte pieces
-        bws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+        bws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(sh), slice_cols, HOTF)
         train_tile = 64 if (dtype == torch.float32 and K > 64) else 128
         granule = train_tile if D % (16 // p_size) == 0 else tile
     else:
@@ -323,14 +337,16 @@ def main():
                                         p(dvals), p(dbias), p(w), w.numel(), flags, None, st()),
                    "flexsae_hier_bwd")
 
-    PRE, REUSE, SWEEP, REDUCE, NO_DW, NO_EPILOGUE = 1, 2, 4, 8, 32, 64
+    PRE, REUSE, SWEEP, REDUCE, NO_DW, NO_EPILOGUE, REUSE_HOT = 1, 2, 4, 8, 32, 64, _lib.BWD_REUSE_HOT_TABLES
     fwd_k_ms = time_kernel_events(torch, lambda: None, fwd_launch, args.steps, args.warmup)
     step_entry_ms = None
     if fused:
         # the API step above went through the fused training-step entry point: time it and its phases
         def train_launch(flags=0):
+            if flags & REUSE:
+                flags |= REUSE_HOT
             _lib.check(lib.flexsae_hier_fwd_bwd(ctypes.byref(sh), p(idx), p(W), p(v), p(b), p(t), p(loss), p(dW),
-                                                DT[dtype], p(dvals), p(dbias), p(bws), bws_bytes, flags, None,
+                                                DT[dtype], p(dvals), p(dbias), p(bws), bws_bytes, flags | HOTF, None,
                                                 st()), "flexsae_hier_fwd_bwd")
 
         step_entry_ms = time_kernel_events(torch, lambda: None, train_launch, args.steps, args.warmup)
@@ -344,7 +360,7 @@ def main():
                            device=dev)
         bwd_k_ms = time_kernel_events(torch, lambda: None, lambda: bwd_launch(0, ubws), args.steps, args.warmup)
         del ubws
-        sweep_name = "hier_train_kernel"
+        sweep_name = "hier_train_hot_kernel" if hot else "hier_train_kernel"
     elif scratch > 0:
         bwd_k_ms = time_kernel_events(torch, lambda: None, bwd_launch, args.steps, args.warmup)
         # the pair list is in the workspace now: time the two phases alone (n_slices launches each)
@@ -382,7 +398,7 @@ def main():
     # workload, the slice budget and the id of the build it was taken on.  A record of another build
     # is not reported as this build's traffic.
     traffic = None
-    traffic_key = f"{args.workload}:{'fused' if staged else scratch >> 20}"
+    traffic_key = f"{args.workload}:{'fused' if staged else slice_w}"  # workload : columns per slice
     traffic_source = None
     traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
     build_id = _lib.build_id()
@@ -445,17 +461,19 @@ def main():
         "build_id": build_id,
         "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
                                f"indices {dist}", "B": B, "K": K, "F": F, "D": D,
-                   "hier_scratch_mb": scratch >> 20, "fused_training_step": bool(fused), "hier_mode": hier_mode,
+                   "hier_scratch_mb": scratch >> 20, "hier_slice_cols": int(slice_w), "hot_latents": hot, "fused_training_step": bool(fused), "hier_mode": hier_mode,
                    "hier_stage_mb": flex.ops.hier_stage_bytes(dev) >> 20},
         "roofline": roofline,
         "step_hbm": {"algorithmic_bytes": abytes["hier_step"],
                      "achieved_GBps": round(gbps(abytes["hier_step"], hier_ms), 1),
-                     "frac_of_peak": round(gbps(abytes["hier_step"], hier_ms) / HBM_PEAK_GBPS, 4)},
+                     "algorithmic_frac_of_peak": round(gbps(abytes["hier_step"], hier_ms) / HBM_PEAK_GBPS, 4),
+                     "note": ALGORITHMIC_NOTE},
         "kernels": {
             "flexsae_hier_fwd (sae_fwd_kernel + loss_finalize)": {
                 "ms": round(fwd_k_ms, 4), "algorithmic_bytes": abytes["fwd_kernel"],
                 "GBps": round(gbps(abytes["fwd_kernel"], fwd_k_ms), 1),
-                "frac_of_peak": round(gbps(abytes["fwd_kernel"], fwd_k_ms) / HBM_PEAK_GBPS, 4)},
+                "algorithmic_frac_of_peak": round(gbps(abytes["fwd_kernel"], fwd_k_ms) / HBM_PEAK_GBPS, 4),
+                "note": ALGORITHMIC_NOTE},
             "flexsae_hier_bwd (pair list + sweep + reduce)": {
                 "ms": round(bwd_k_ms, 4), "algorithmic_bytes": abytes["hier_bwd_kernel"],
                 "GBps": round(gbps(abytes["hier_bwd_kernel"], bwd_k_ms), 1)},

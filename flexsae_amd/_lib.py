@@ -8,9 +8,10 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libflexsae_amd.so")
+# FLEXSAE_AMD_LIBRARY names another build of the library to load instead of the in-tree one
+LIB_PATH = os.environ.get("FLEXSAE_AMD_LIBRARY") or os.path.join(_HERE, "libflexsae_amd.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # flexsae_status
 OK = 0
@@ -32,6 +33,9 @@ BWD_REDUCE_ONLY = 8
 BWD_SCALE_BY_GRAD_OUT = 16
 BWD_NO_DW = 32
 BWD_SKIP_EPILOGUE = 64
+BWD_HOT_LATENTS = 128
+BWD_HOT_NO_HEADROOM = 512
+BWD_REUSE_HOT_TABLES = 1024
 TOPK_BWD_FP32_RESIDUAL = 256
 
 
@@ -79,6 +83,10 @@ SIGNATURES = {
     "flexsae_topk_bwd": (_int, [_shape_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _sz, _int, _p]),
     "flexsae_topk_bwd_workspace_bytes": (_sz, [_shape_p, _i64]),
     "flexsae_cast_from_f32": (_int, [_p, _int, _p, _i64, _p]),
+    "flexsae_scale_from_f32": (_int, [_p, _int, _p, _i64, _p, _p]),
+    "flexsae_hier_hot_latents_supported": (_int, [_shape_p]),
+    "flexsae_hier_hot_stats": (_int, [_shape_p, _p, _p, _p]),
+    "flexsae_hier_fwd_bwd_workspace_bytes_flags": (_sz, [_shape_p, _i64, _int]),
 }
 
 _lib = None

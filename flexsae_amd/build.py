@@ -10,6 +10,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libflexsae_amd.so")
 
+# gfx950 only: some kernels use more LDS per workgroup than the 64 KiB of earlier gfx9 parts
+# (csr_sort_long_kernel 65 600 bytes, the hot-latent variant of the training-step kernel more), the
+# gfx950 lane-swap and bf16 conversion instructions, and buffer loads with the LDS as destination.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

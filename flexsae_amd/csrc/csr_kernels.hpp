@@ -204,6 +204,9 @@ __device__ __forceinline__ void block_bitonic_sort(Ptr a, uint32_t n) {
 // would cost several times more.
 constexpr uint32_t kSortLdsElems = 8192;
 constexpr uint32_t kSortRowsMax = 8192;  // rows (B) the counting sort has LDS counters for
+// buf + rowcnt + wave_tot come to 65 600 bytes of LDS per block: more than the 64 KiB of earlier gfx9
+// parts, within the 160 KiB a workgroup may use on gfx950 (the only target of this library)
+static_assert((kSortLdsElems + kSortRowsMax + 1024 / kWave) * 4 <= 160 * 1024, "LDS of csr_sort_long_kernel");
 __global__ __launch_bounds__(1024) void csr_sort_long_kernel(const uint32_t *__restrict__ begin,
                                                             uint32_t *__restrict__ map,
                                                             const uint32_t *__restrict__ long_count,
@@ -563,19 +566,23 @@ __global__ void fill_f32_kernel(float *__restrict__ p, int64_t n) {
     p[i] = 0.f;
 }
 
+// dst = GT(src * scale[0]) (scale null: a plain cast)
 template <typename GT>
 __global__ void cast_from_f32_kernel(void *__restrict__ dst, const float *__restrict__ src,
-                                     int64_t n) {
+                                     int64_t n, const float *__restrict__ scale = nullptr) {
+  const float g = scale ? scale[0] : 1.0f;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t n4 = n >> 2;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) {
     float x[4];
     load_vec<float, 4>(src, i * 4, x);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) x[k] *= g;
     store_vec<GT, 4>(dst, i * 4, x);
   }
   for (int64_t i = (n4 << 2) + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
        i += stride) {
-    float x[1] = {src[i]};
+    float x[1] = {src[i] * g};
     store_vec<GT, 1>(dst, i, x);
   }
 }

@@ -10,6 +10,7 @@
 #include "csr_kernels.hpp"
 #include "hier_bwd_kernels.hpp"
 #include "hier_train_kernel.hpp"
+#include "hier_hot_kernel.hpp"
 #include "segment_kernels.hpp"
 #include "topk_bwd_kernels.hpp"
 
@@ -48,6 +49,7 @@ constexpr int kBlock = 256;              // threads per block of the wave-per-it
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr size_t kAlign = 256;
 constexpr int kBwdSgdUpdate = 1 << 20;  // internal flag of the slice loop: dW is the weight matrix, updated in place
+constexpr int kBwdHot = 1 << 21;        // internal flag of the slice loop: hot latents are accumulated in the LDS
 constexpr unsigned kLongBlocks = 1024;    // leading blocks of a reduction launch that serve hot latents
 
 inline bool valid_dtype(int d) { return d == FLEXSAE_F32 || d == FLEXSAE_BF16 || d == FLEXSAE_F16; }
@@ -393,9 +395,22 @@ struct HierBwdPlan {
   size_t off_begin, off_map, off_slot, off_csr, off_chunk, off_cls, off_cls_list, off_sfinal, off_colsum, off_loss, off_dvpart, off_partial;  // per-slice buffers follow
   size_t n_loss_partials;  // training-step kernel: one per (tile of 64 or 128 columns, row)
   size_t fixed_bytes;      // everything that does not depend on the slice width
+  // hot-latent tables (only with `hot`): slots with the hot pairs marked, control words, the hot
+  // latents, the candidates and what became of them, the long latents that stayed cold and their
+  // chunk table
+  bool hot;
+  size_t off_hslot, off_hot_ctrl, off_hot_list, off_cand_list, off_cand_state, off_long_cand, off_long2, off_chunk2;
+  size_t n_row_blocks;     // blocks of kHotRowsPerBlock rows
 };
 
-HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
+// Hot-latent accumulators: 16-bit weights of at most 64 steps (one register per row piece, four
+// wavefronts per SIMD next to 144 KiB of accumulators) whose slices the piece reduction serves.
+inline bool hot_supported(const flexsae_shape *s) {
+  return s->D % 4 == 0 && s->K <= 64 && s->weight_dtype != FLEXSAE_F32 &&
+         s->D % (s->weight_dtype == FLEXSAE_BF16 ? 8 : 4) == 0 && s->B * s->K < (1LL << 31);
+}
+
+HierBwdPlan plan_hier_bwd(const flexsae_shape *s, bool hot = false) {
   HierBwdPlan p;
   p.vec = (s->D % 4 == 0) ? 4 : (s->D % 2 == 0) ? 2 : 1;
   p.tile = kWave * p.vec;
@@ -433,6 +448,27 @@ HierBwdPlan plan_hier_bwd(const flexsae_shape *s) {
   p.off_dvpart = off;
   const int64_t tt = train_tile_cols(s);
   off += round_up(static_cast<size_t>(p.d_pad / (p.tile < tt ? p.tile : tt)) * p.n_pairs * 4, kAlign);
+  p.hot = hot;
+  p.n_row_blocks = static_cast<size_t>(ceil_div(s->B, kHotRowsPerBlock));
+  if (hot) {
+    const size_t n_long_max = p.n_pairs / 65 + 2;
+    p.off_hslot = off;
+    off += round_up(p.n_pairs * 4, kAlign);
+    p.off_hot_ctrl = off;
+    off += round_up(kHotCtrlWords * 4, kAlign);
+    p.off_hot_list = off;
+    off += round_up(kHotMax * 4, kAlign);
+    p.off_cand_list = off;
+    off += round_up(kHotMax * 4, kAlign);
+    p.off_cand_state = off;
+    off += round_up(kHotMax * 4, kAlign);
+    p.off_long_cand = off;
+    off += round_up(n_long_max * 4, kAlign);
+    p.off_long2 = off;
+    off += round_up(n_long_max * 4, kAlign);
+    p.off_chunk2 = off;
+    off += round_up(n_long_max * 4, kAlign);
+  }
   p.off_partial = off;
   p.fixed_bytes = off;
   return p;
@@ -543,14 +579,56 @@ void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const in
 #undef FLEXSAE_TRAIN
 }
 
+// The training-step kernel with hot-latent accumulators (16-bit weights, K <= 64): one block per
+// (row block, 128-column tile); every block first takes its share of the previous slice's second steps.
+template <typename WT, typename PT>
+void launch_train_hot_kernel(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
+                             const void *weight, const void *vals, float coef, const uint32_t *hslot, void *P,
+                             float *dvals, float *s_final, int d_pad, float *loss_partial, int *status_flag,
+                             int64_t cols, int col0, int slice_w, hipStream_t st, HotFinalize fin,
+                             const HotBlockFinalize &hfin, uint32_t *ctrl, float *hot_partial,
+                             int n_row_blocks, int headroom) {
+  if constexpr (sizeof(typename Traits<WT>::store_t) == 2) {
+    const int n_tiles = static_cast<int>(cols / kHotCols);
+    const unsigned grid = static_cast<unsigned>(n_tiles) * static_cast<unsigned>(n_row_blocks);
+    if (fin.mode != 0) fin.n_blocks = grid;  // every block takes a share
+#define FLEXSAE_TRAIN_HOT(KM)                                                                                   \
+  do {                                                                                                          \
+    const auto kernel = s->K == KM ? hier_train_hot_kernel<WT, PT, KM, true> : hier_train_hot_kernel<WT, PT, KM, false>; \
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kHotThreads), 0, st, indices, weight, vals, s->vals_dtype, ta.bias, \
+                       s->bias_dtype, ta.target, s->target_dtype, coef, hslot, P, dvals, s_final, d_pad,        \
+                       loss_partial, status_flag, s->B, n_tiles, n_row_blocks, col0, slice_w,                   \
+                       static_cast<int>(s->K), s->F, static_cast<int>(s->D), ctrl, hot_partial, headroom, fin, hfin); \
+  } while (0)
+    if (s->K <= 16) {
+      FLEXSAE_TRAIN_HOT(16);
+    } else if (s->K <= 32) {
+      FLEXSAE_TRAIN_HOT(32);
+    } else {
+      FLEXSAE_TRAIN_HOT(64);
+    }
+#undef FLEXSAE_TRAIN_HOT
+  }
+}
+
 // per-slice buffers after the fixed part: chunk partials[n_partial_rows, w] | P[B*K, w]
 size_t hier_partial_bytes(const HierBwdPlan &p, int64_t slice_w) {
   return round_up(p.n_partial_rows * static_cast<size_t>(slice_w) * 4, kAlign);
 }
 
+size_t hier_p_bytes(const HierBwdPlan &p, int64_t slice_w) {
+  return round_up(p.n_pairs * static_cast<size_t>(slice_w) * p.p_size, kAlign);
+}
+
+// one buffer of block partials of the hot latents: [tiles of the slice][row blocks][kHotMax][128] fp32
+size_t hier_hot_partial_bytes(const HierBwdPlan &p, int64_t slice_w) {
+  return round_up(static_cast<size_t>(ceil_div(slice_w, kHotCols)) * p.n_row_blocks * kHotMax * kHotCols * 4, kAlign);
+}
+
+// ... | chunk partials | P | (hot: two buffers of block partials, used by alternate slices)
 size_t hier_bwd_bytes(const HierBwdPlan &p, int64_t slice_w) {
-  return p.fixed_bytes + hier_partial_bytes(p, slice_w) +
-         round_up(p.n_pairs * static_cast<size_t>(slice_w) * p.p_size, kAlign);
+  return p.fixed_bytes + hier_partial_bytes(p, slice_w) + hier_p_bytes(p, slice_w) +
+         (p.hot ? 2 * hier_hot_partial_bytes(p, slice_w) : 0);
 }
 
 // Segment reduction of one slice plus the finalize step of its hot latents.  fp32 contributions
@@ -650,6 +728,23 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   const bool narrow_reduce = s->B * s->K >= 4 * s->F;
   float *partial = reinterpret_cast<float *>(ws + pl.off_partial);
   void *P = ws + pl.off_partial + hier_partial_bytes(pl, slice_w);
+  // Hot latents (training step only): their pairs are marked in hslot and accumulated by the
+  // training-step kernel; the chunked part of the reduction then serves the long latents that stayed
+  // cold, from a list and a chunk table of their own.
+  const bool hot = (flags & kBwdHot) != 0 && pl.hot && train != nullptr;
+  uint32_t *hot_ctrl = hot ? reinterpret_cast<uint32_t *>(ws + pl.off_hot_ctrl) : nullptr;
+  const uint32_t *hot_list = hot ? reinterpret_cast<const uint32_t *>(ws + pl.off_hot_list) : nullptr;
+  float *hot_partial[2] = {nullptr, nullptr};
+  CsrScratch sc_cold = sc;  // the long latents the reduction serves
+  if (hot) {
+    uint8_t *base = static_cast<uint8_t *>(P) + hier_p_bytes(pl, slice_w);
+    hot_partial[0] = reinterpret_cast<float *>(base);
+    hot_partial[1] = reinterpret_cast<float *>(base + hier_hot_partial_bytes(pl, slice_w));
+    sc_cold.long_count = hot_ctrl + kHotLong2Count;
+    sc_cold.long_list = reinterpret_cast<uint32_t *>(ws + pl.off_long2);
+    chunk_begin = reinterpret_cast<uint32_t *>(ws + pl.off_chunk2);
+  }
+  const int hot_headroom = (flags & FLEXSAE_BWD_HOT_NO_HEADROOM) ? -6 : 2;
   // columns that are worked on: whole reduction tiles, or, with the piece reduction, whole training
   // tiles (tiles that lie entirely beyond column D are left out, and so are their shares below)
   const int64_t d_used = hier_cols_used(s, pl, train != nullptr, piece != 0);
@@ -671,11 +766,21 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   // training-step launch (a gradient of the weight's own dtype only: that is what that kernel writes);
   // the last slice's gets a launch of its own.
   HotFinalize pending = {};
+  HotBlockFinalize pending_hot = {};
   const bool fold = std::is_same<GT, WT>::value && train != nullptr && do_sweep && do_reduce;
-  for (int64_t col0 = 0; col0 < s->D; col0 += slice_w) {
+  int slice_no = 0;
+  for (int64_t col0 = 0; col0 < s->D; col0 += slice_w, ++slice_no) {
     const int64_t cols = (d_used - col0) < slice_w ? (d_used - col0) : slice_w;
     const int tps = static_cast<int>(cols / pl.tile);
-    if (train && do_sweep) {
+    if (train && do_sweep && hot) {
+      launch_train_hot_kernel<WT, PT>(s, *train, indices, weight, vals, coef,
+                                      reinterpret_cast<const uint32_t *>(ws + pl.off_hslot), P, dv_part, s_final, d_pad,
+                                      reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
+                                      static_cast<int>(col0), sw, st, pending, pending_hot, hot_ctrl,
+                                      hot_partial[slice_no & 1], static_cast<int>(pl.n_row_blocks), hot_headroom);
+      pending = HotFinalize{};
+      pending_hot = HotBlockFinalize{};
+    } else if (train && do_sweep) {
       launch_train_kernel_k<WT, PT>(s, *train, indices, weight, vals, coef, slot, P, dv_part, s_final, d_pad,
                                     reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
                                     static_cast<int>(col0), sw, st, pending);
@@ -705,14 +810,27 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     const bool cache_sized = static_cast<size_t>(s->B * s->K) * static_cast<size_t>(sw) * pl.p_size <= (size_t{384} << 20);
     const bool by_pieces =
         piece != 0 && (update || cols % pl.tile != 0 || s->B * s->K <= 2 * s->F || cache_sized);
-    launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
+    launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc_cold, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
                                    static_cast<int>(col0), sw, D, st, by_pieces ? piece : 0, cols, s->B * s->K, update,
                                    sparse ? cls_begin : nullptr, sparse ? cls_list : nullptr, fold ? &pending : nullptr);
+    if (hot) {
+      // the block partials of the slice's hot latents are added up by the next training-step launch
+      // (they live in the buffer that launch does not write), or here
+      const HotBlockFinalize h = {hot_ctrl, hot_list, hot_partial[slice_no & 1], dW, dw_scale,
+                                  static_cast<int>(cols / kHotCols), static_cast<int>(pl.n_row_blocks),
+                                  static_cast<int>(col0), D, update};
+      if (fold)
+        pending_hot = h;
+      else
+        hipLaunchKernelGGL((hot_block_finalize_kernel<GT>), dim3(256), dim3(kBlock), 0, st, h);
+    }
   }
   if (pending.n_blocks != 0) {
     pending.n_blocks = 256u;
     hipLaunchKernelGGL((hot_finalize_kernel<GT>), dim3(pending.n_blocks), dim3(kBlock), 0, st, pending);
   }
+  if (pending_hot.ctrl != nullptr)
+    hipLaunchKernelGGL((hot_block_finalize_kernel<GT>), dim3(256), dim3(kBlock), 0, st, pending_hot);
   if (!do_sweep) return;
   if (!do_reduce && !train) return;  // measurement aid of the plain backward: sweep kernels only
   if (flags & FLEXSAE_BWD_SKIP_EPILOGUE) return;
@@ -791,6 +909,31 @@ void finish_pair_list(const flexsae_shape *s, const HierBwdPlan &pl, uint8_t *ws
                      reinterpret_cast<uint32_t *>(ws + pl.off_cls_list));
 }
 
+// Hot-latent tables of a workspace whose pair list is complete: the slots with the hot pairs marked,
+// the hot latents, the long latents that stayed cold and their chunk table.
+void build_hot_tables(const flexsae_shape *s, const HierBwdPlan &pl, uint8_t *ws, const CsrScratch &sc, hipStream_t st) {
+  const uint32_t *begin = reinterpret_cast<const uint32_t *>(ws + pl.off_begin);
+  const uint32_t *map = reinterpret_cast<const uint32_t *>(ws + pl.off_map);
+  uint32_t *hslot = reinterpret_cast<uint32_t *>(ws + pl.off_hslot);
+  uint32_t *ctrl = reinterpret_cast<uint32_t *>(ws + pl.off_hot_ctrl);
+  uint32_t *hot_list = reinterpret_cast<uint32_t *>(ws + pl.off_hot_list);
+  uint32_t *cand_list = reinterpret_cast<uint32_t *>(ws + pl.off_cand_list);
+  uint32_t *cand_state = reinterpret_cast<uint32_t *>(ws + pl.off_cand_state);
+  uint32_t *long_cand = reinterpret_cast<uint32_t *>(ws + pl.off_long_cand);
+  uint32_t *long2 = reinterpret_cast<uint32_t *>(ws + pl.off_long2);
+  const int64_t n_pairs = s->B * s->K;
+  hipLaunchKernelGGL(copy_u32_kernel, dim3(grid_for(n_pairs, 256, 8192)), dim3(256), 0, st, hslot,
+                     reinterpret_cast<const uint32_t *>(ws + pl.off_slot), n_pairs);
+  hipLaunchKernelGGL(hot_select_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count, sc.long_list, ctrl,
+                     cand_list, long_cand, static_cast<uint32_t>(kHotMax));
+  hipLaunchKernelGGL(hot_mark_kernel, dim3(kHotMax), dim3(256), 0, st, begin, map, ctrl, cand_list, cand_state,
+                     hot_list, hslot, static_cast<uint32_t>(s->K));
+  hipLaunchKernelGGL(hot_cold_long_kernel, dim3(64), dim3(256), 0, st, sc.long_count, sc.long_list, long_cand,
+                     cand_state, ctrl, long2);
+  hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, ctrl + kHotLong2Count, long2,
+                     reinterpret_cast<uint32_t *>(ws + pl.off_chunk2), static_cast<uint32_t *>(nullptr), 0);
+}
+
 // ---- TopK backward: workspace plan and slice loop ---------------------------------------
 
 struct TopkBwdPlan {
@@ -805,7 +948,8 @@ TopkBwdPlan plan_topk_bwd(const flexsae_shape *s, int flags = 0) {
   TopkBwdPlan p;
   // The reference hands its backward the residual gradient in the weight dtype
   // (topk_kernels.py:52,221); for bf16 weights the gathers here read a bf16 copy as well, unless
-  // the caller asks for the fp32 residual (the workspace layout of that variant is a subset).
+  // the caller asks for the fp32 residual (no copy, but narrower tiles and so more per-tile dvals
+  // shares: flexsae_topk_bwd_workspace_bytes returns the larger of the two layouts).
   p.resid16 = FLEXSAE_TOPK_RESID16 && s->weight_dtype == FLEXSAE_BF16 && !(flags & FLEXSAE_TOPK_BWD_FP32_RESIDUAL);
   p.vec = (s->D % 4 == 0) ? 4 : (s->D % 2 == 0) ? 2 : 1;
   // all-bf16: 16 bytes per lane (512-column tiles) halve the per-tile overheads
@@ -1026,13 +1170,37 @@ size_t flexsae_hier_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_co
   return hier_bwd_bytes(pl, sw);
 }
 
-size_t flexsae_hier_fwd_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_cols) {
+size_t flexsae_hier_fwd_bwd_workspace_bytes_flags(const flexsae_shape *s, int64_t slice_cols, int flags) {
   if (check_shape(s) != FLEXSAE_OK || !train_supported(s)) return 0;
-  const HierBwdPlan pl = plan_hier_bwd(s);
+  const bool hot = (flags & FLEXSAE_BWD_HOT_LATENTS) && hot_supported(s);
+  const HierBwdPlan pl = plan_hier_bwd(s, hot);
   const int64_t granule = piece_reduce_ok(s, pl, nullptr, s->weight_dtype) ? train_tile_cols(s) : pl.tile;
   int64_t sw = slice_cols <= 0 ? granule : ceil_div(slice_cols, granule) * granule;
   if (sw > pl.d_pad) sw = pl.d_pad;
   return hier_bwd_bytes(pl, sw);
+}
+
+size_t flexsae_hier_fwd_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_cols) {
+  return flexsae_hier_fwd_bwd_workspace_bytes_flags(s, slice_cols, 0);
+}
+
+int flexsae_hier_hot_latents_supported(const flexsae_shape *s) {
+  return check_shape(s) == FLEXSAE_OK && train_supported(s) && hot_supported(s) ? 1 : 0;
+}
+
+int flexsae_hier_hot_stats(const flexsae_shape *s, const void *workspace, uint32_t *stats, void *stream) {
+  const int rc = check_shape(s);
+  if (rc != FLEXSAE_OK) return rc;
+  if (!workspace || !stats) return FLEXSAE_ERR_INVALID_ARGUMENT;
+  if (!train_supported(s) || !hot_supported(s)) return FLEXSAE_ERR_UNSUPPORTED;
+  if (!aligned(workspace, kAlign) || !aligned(stats, 4)) return FLEXSAE_ERR_ALIGNMENT;
+  const HierBwdPlan pl = plan_hier_bwd(s, true);
+  const uint32_t *ctrl = reinterpret_cast<const uint32_t *>(static_cast<const uint8_t *>(workspace) + pl.off_hot_ctrl);
+  static_assert(kHotNHot == 0 && kHotNCand == 1 && kHotLong2Count == 2 && kHotThreshold == 3 && kHotDeferred == 4,
+                "flexsae_hier_hot_stats hands out the first five control words");
+  hipLaunchKernelGGL(copy_u32_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), stats, ctrl,
+                     static_cast<int64_t>(5));
+  return launch_status();
 }
 
 int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void *weight,
@@ -1156,7 +1324,11 @@ int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void
       (!defer_reduce && !no_dw && (!dW || !valid_dtype(dW_dtype))))
     return FLEXSAE_ERR_INVALID_ARGUMENT;
   if (!train_supported(s)) return FLEXSAE_ERR_UNSUPPORTED;
-  const HierBwdPlan pl = plan_hier_bwd(s);  // D % 4 == 0 here, so tiles are 256 columns
+  // hot-latent accumulators: a hint, taken where the shape allows them, the reductions run in this
+  // call and every pointer is aligned for the piece reduction (the workspace layout depends on it)
+  const bool hot = (flags & FLEXSAE_BWD_HOT_LATENTS) && hot_supported(s) && !defer_reduce &&
+                   piece_reduce_ok(s, plan_hier_bwd(s), (defer_reduce || no_dw) ? nullptr : dW, dW_dtype);
+  const HierBwdPlan pl = plan_hier_bwd(s, hot);  // D % 4 == 0 here, so tiles are 256 columns
   if (!aligned(indices, 8) || !aligned(weight, 4 * dtype_size(s->weight_dtype)) ||
       !aligned(vals, dtype_size(s->vals_dtype)) || !aligned(bias, 2 * dtype_size(s->bias_dtype)) ||
       !aligned(target, 2 * dtype_size(s->target_dtype)) || !aligned(loss, 4) ||
@@ -1184,6 +1356,8 @@ int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void
                      status_flag, st);
     finish_pair_list(s, pl, ws, begin, sc, st);
   }
+  if (hot && !((flags & FLEXSAE_BWD_REUSE_PAIR_LIST) && (flags & FLEXSAE_BWD_REUSE_HOT_TABLES)))
+    build_hot_tables(s, pl, ws, sc, st);
   const double count = static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D);
   const float coef = static_cast<float>(2.0 / count);
   const TrainArgs ta = {bias, target, loss, s->B * (hier_cols_used(s, pl, true, piece) / train_tile_cols(s)),
@@ -1191,8 +1365,9 @@ int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void
   // without dW the reductions are left out like in the deferred case (dW_dtype only selects a template then)
   launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, sgd_step, coef, dW,
                           no_dw ? s->weight_dtype : dW_dtype, dvals, dbias, ws,
-                          (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE)) |
-                              (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0) | (sgd_step ? kBwdSgdUpdate : 0),
+                          (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE |
+                                    FLEXSAE_BWD_HOT_NO_HEADROOM)) |
+                              (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0) | (sgd_step ? kBwdSgdUpdate : 0) | (hot ? kBwdHot : 0),
                           status_flag, st, &ta, piece ? static_cast<int>(piece_cols(pl)) : 0);
   return launch_status();
 }
@@ -1206,7 +1381,7 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *s, const int64_t *indices, const v
                          void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
                          size_t workspace_bytes, int flags, int *status_flag, void *stream) {
   return hier_fwd_bwd_impl(s, indices, weight, vals, bias, target, loss, dW, dW_dtype, dvals, dbias, workspace,
-                           workspace_bytes, flags & ~kBwdSgdUpdate, status_flag, stream, nullptr);
+                           workspace_bytes, flags & ~(kBwdSgdUpdate | kBwdHot), status_flag, stream, nullptr);
 }
 
 int flexsae_hier_sgd_step(const flexsae_shape *s, const int64_t *indices, void *weight, const void *vals,
@@ -1215,8 +1390,10 @@ int flexsae_hier_sgd_step(const flexsae_shape *s, const int64_t *indices, void *
                           int *status_flag, void *stream) {
   if (!step || !s) return FLEXSAE_ERR_INVALID_ARGUMENT;
   return hier_fwd_bwd_impl(s, indices, weight, vals, bias, target, loss, weight, s->weight_dtype, dvals, dbias,
-                           workspace, workspace_bytes, flags & FLEXSAE_BWD_REUSE_PAIR_LIST, status_flag, stream,
-                           step);
+                           workspace, workspace_bytes,
+                           flags & (FLEXSAE_BWD_REUSE_PAIR_LIST | FLEXSAE_BWD_HOT_LATENTS | FLEXSAE_BWD_REUSE_HOT_TABLES |
+                                    FLEXSAE_BWD_HOT_NO_HEADROOM),
+                           status_flag, stream, step);
 }
 
 int flexsae_scale(void *dst, const void *src, int dtype, int64_t n, const float *scale, void *stream) {
@@ -1261,10 +1438,18 @@ int flexsae_csr_build(const int64_t *indices, int64_t B, int64_t K, int64_t F, u
 
 size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *s, int64_t slice_cols) {
   if (check_shape(s) != FLEXSAE_OK) return 0;
-  const TopkBwdPlan pl = plan_topk_bwd(s);
-  int64_t sw = slice_cols <= 0 ? pl.tile : ceil_div(slice_cols, pl.tile) * pl.tile;
-  if (sw > pl.d_pad) sw = pl.d_pad;
-  return topk_bwd_bytes(pl, sw);
+  // The query takes no flags, so it covers both layouts of the call: the bf16-residual one (wide
+  // tiles plus the bf16 copy of the residual) and the FLEXSAE_TOPK_BWD_FP32_RESIDUAL one (narrower
+  // tiles: twice the per-tile dvals shares, which outweighs the copy once K exceeds 256).
+  size_t need = 0;
+  for (const int flags : {0, static_cast<int>(FLEXSAE_TOPK_BWD_FP32_RESIDUAL)}) {
+    const TopkBwdPlan pl = plan_topk_bwd(s, flags);
+    int64_t sw = slice_cols <= 0 ? pl.tile : ceil_div(slice_cols, pl.tile) * pl.tile;
+    if (sw > pl.d_pad) sw = pl.d_pad;
+    const size_t bytes = topk_bwd_bytes(pl, sw);
+    if (bytes > need) need = bytes;
+  }
+  return need;
 }
 
 int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32_t *map,
@@ -1343,23 +1528,28 @@ int flexsae_topk_bwd(const flexsae_shape *s, const uint32_t *begin, const uint32
   return launch_status();
 }
 
-int flexsae_cast_from_f32(void *dst, int dst_dtype, const float *src, int64_t n, void *stream) {
+int flexsae_scale_from_f32(void *dst, int dst_dtype, const float *src, int64_t n, const float *scale,
+                           void *stream) {
   if (!dst || !src || n < 0 || !valid_dtype(dst_dtype)) return FLEXSAE_ERR_INVALID_ARGUMENT;
   if (n == 0) return FLEXSAE_OK;
-  if (!aligned(src, 16) || !aligned(dst, 4 * dtype_size(dst_dtype))) return FLEXSAE_ERR_ALIGNMENT;
+  if (!aligned(src, 16) || !aligned(dst, 4 * dtype_size(dst_dtype)) || !aligned(scale, 4)) return FLEXSAE_ERR_ALIGNMENT;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(grid_for(ceil_div(n, 4), 256, 1 << 16));
   switch (dst_dtype) {
     case FLEXSAE_F32:
-      hipLaunchKernelGGL(cast_from_f32_kernel<float>, grid, dim3(256), 0, st, dst, src, n);
+      hipLaunchKernelGGL(cast_from_f32_kernel<float>, grid, dim3(256), 0, st, dst, src, n, scale);
       break;
     case FLEXSAE_BF16:
-      hipLaunchKernelGGL(cast_from_f32_kernel<bf16_t>, grid, dim3(256), 0, st, dst, src, n);
+      hipLaunchKernelGGL(cast_from_f32_kernel<bf16_t>, grid, dim3(256), 0, st, dst, src, n, scale);
       break;
     default:
-      hipLaunchKernelGGL(cast_from_f32_kernel<f16_t>, grid, dim3(256), 0, st, dst, src, n);
+      hipLaunchKernelGGL(cast_from_f32_kernel<f16_t>, grid, dim3(256), 0, st, dst, src, n, scale);
   }
   return launch_status();
+}
+
+int flexsae_cast_from_f32(void *dst, int dst_dtype, const float *src, int64_t n, void *stream) {
+  return flexsae_scale_from_f32(dst, dst_dtype, src, n, nullptr, stream);
 }
 
 }  // extern "C"

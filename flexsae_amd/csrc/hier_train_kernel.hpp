@@ -99,8 +99,14 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   }
   const int64_t item = static_cast<int64_t>(blockIdx.x - fin.n_blocks) * (blockDim.x >> 6) + wave_in_block();
   if (item >= n_items) return;  // uniform per wavefront
+#ifdef FLEXSAE_TRAIN_ROW_MAJOR
+  const int n_t = static_cast<int>(n_items / B);
+  const int64_t b = item / n_t;
+  const int t = static_cast<int>(item - b * n_t);
+#else
   const int t = static_cast<int>(item / B);
   const int64_t b = item - static_cast<int64_t>(t) * B;
+#endif
   const int pc = t * (kWave * VEC) + lane * VEC;  // column inside the slice
   const int d0 = col0 + pc;
   const bool active = d0 < D;
@@ -153,23 +159,29 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   const uint32_t w_lane_bytes = static_cast<uint32_t>(d0) * sizeof(S_t);  // beyond the row if !active
   {
     const int kb = k_bound();
+    if constexpr (LDSROWS > 0) {
+      // The loads into the LDS first, in a loop of their own, then a scheduling barrier: the wait
+      // below counts on every one of them having been issued before the first register gather,
+      // and nothing else orders the two kinds of load (they carry no dependence on each other).
 #pragma unroll
-    for (int k = 0; k < KMAX; ++k) {
+      for (int k = 0; k < LDSROWS; ++k) {
+        const uint32_t row = static_cast<uint32_t>(bcast_i32(my_row[k / kWave], k % kWave));
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            row_descriptor(weight, row, w_row_bytes),
+            (__attribute__((address_space(3))) void *)(my_lds + k * kWave),
+            4, w_lane_bytes, 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int k = LDSROWS; k < KMAX; ++k) {
       if (FULL || k < kb) {  // uniform
         const uint32_t row = static_cast<uint32_t>(bcast_i32(my_row[k / kWave], k % kWave));
-        if constexpr (LDSROWS > 0) {
-          if (k < LDSROWS) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                row_descriptor(weight, row, w_row_bytes),
-                (__attribute__((address_space(3))) void *)(my_lds + k * kWave),
-                4, w_lane_bytes, 0, 0, 0);
-            continue;
-          }
-        }
         const auto dw = descriptor_load<sizeof(raw_t)>(row_descriptor(weight, row, w_row_bytes), w_lane_bytes);
         __builtin_memcpy(&raw[k], &dw, sizeof(raw_t));
       }
     }
+    if constexpr (LDSROWS > 0) __builtin_amdgcn_sched_barrier(0);  // no gather sinks below the wait either
   }
 
 

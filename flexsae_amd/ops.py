@@ -8,7 +8,7 @@ Op graph (names under the ``flexsae_amd::`` namespace):
     topk_bwd(grad_out, indices, weight, vals, resid) -> (dW, dvals, dbias)
     hier_train_sliced(indices, weight, vals, bias, target) -> (loss, dvals, dbias, dW)   [unit gradient]
     scale_(x, grad_out), scale_by(x, grad_out) -> x * grad_out
-    hier_train(indices, weight, vals, bias, target) -> (loss, dvals, dbias, stage)       [unit gradient]
+    hier_train(indices, weight, vals, bias, target, stage) -> (loss, dvals, dbias)       [unit gradient; fills stage]
     hier_finish(grad_out, indices, weight, vals, stage) -> dW
 
 ``resid[B,D]`` (fp32) is the reconstruction error of the full row, the only state the first four
@@ -173,39 +173,114 @@ topk_fwd.register_fake(_fwd_fake)
 
 
 # Scratch the hierarchical backward may use for the per-pair contributions of one slice of D
-# columns.  More scratch = wider slices = fewer passes; 0 selects the atomic single-pass fallback.
-_hier_scratch_bytes = int(os.environ.get("FLEXSAE_HIER_SCRATCH_MB", "256")) << 20
+# columns.  More scratch = wider slices = fewer passes; 0 selects the atomic single-pass fallback;
+# None (the default) sizes it from the problem, see _hier_scratch_budget.
+_hier_scratch_bytes = (int(os.environ["FLEXSAE_HIER_SCRATCH_MB"]) << 20) if "FLEXSAE_HIER_SCRATCH_MB" in os.environ else None
+_HIER_SCRATCH_CAP = 256 << 20
 
 
-# Narrowest slice the scratch budget may lead to on its own: slices below 256 columns run slower
-# (more launches, each too short to overlap its gather, arithmetic and store phases), so a budget
-# that gives fewer columns is exceeded up to this width unless `set_hier_min_slice_cols` lowers it.
-_hier_min_slice_cols = int(os.environ.get("FLEXSAE_HIER_MIN_SLICE_COLS", "256"))
+# Narrowest slice the scratch budget may lead to on its own; a budget that gives fewer columns is
+# exceeded up to this width.  None (the default): 256 columns -- narrower slices measured slower at
+# B*K = 2^19 pairs of bf16 rows (more launches, each too short to overlap its gather, arithmetic
+# and store phases) -- except for fp32 rows of more than 64 steps, whose training-step kernel works
+# on 64-column tiles and measured fastest one tile at a time (B = 2048, K = 256: 1.20 ms with
+# 64-column slices, 1.25 with 128, 1.22 with 256).
+_hier_min_slice_cols = (int(os.environ["FLEXSAE_HIER_MIN_SLICE_COLS"])
+                        if "FLEXSAE_HIER_MIN_SLICE_COLS" in os.environ else None)
 
 
-def set_hier_min_slice_cols(cols: int) -> None:
-    """Narrowest column slice of the sliced hierarchical step (default 256).  128 (16-bit weights)
-    halves the scratch of large problems at a cost of 5-10 % of the step time."""
+def set_hier_min_slice_cols(cols) -> None:
+    """Narrowest column slice of the sliced hierarchical step (``None``: 256, or 64 for fp32 rows of
+    more than 64 steps).  128 (16-bit weights) halves the scratch of large problems at a cost of
+    5-10 % of the step time."""
     global _hier_min_slice_cols
-    _hier_min_slice_cols = max(1, int(cols))
+    _hier_min_slice_cols = None if cols is None else max(1, int(cols))
 
 
-def _hier_scratch_budget(K: int) -> int:
-    return _hier_scratch_bytes
+def _train_tile_cols(K: int, weight_dtype) -> int:
+    """Columns per tile of the training-step kernel (train_tile_cols() of the library)."""
+    return 64 if (weight_dtype == torch.float32 and K > 64) else 128
 
 
-def _hier_slice_cols(B: int, K: int, p_size: int) -> int:
-    return max(_hier_min_slice_cols, _hier_scratch_budget(K) // (B * K * p_size), 1)
+def _hier_scratch_budget(B: int, K: int, F: int, D: int, weight_dtype) -> int:
+    """Bytes the contributions of one slice may take.  Unless set explicitly: 0.45 of the weight
+    matrix, at most 256 MiB -- memory above the inputs then stays within about 1.25 of the TopK
+    loss's (whose peak is the dense gradient plus the residual) whatever K is, at 4-5 % of the step
+    time where that is less than the 256 MiB that measured fastest (B = 4096, F = 65536, D = 2304,
+    bf16: K = 32 0.483 instead of 0.463 ms, K = 64 0.751 instead of 0.717 ms; K = 128 unchanged)."""
+    if _hier_scratch_bytes is not None:
+        return _hier_scratch_bytes
+    sw = 4 if weight_dtype == torch.float32 else 2
+    return min(_HIER_SCRATCH_CAP, int(0.45 * F * D * sw))
+
+
+def _hier_slice_cols(B: int, K: int, F: int, D: int, weight_dtype) -> int:
+    p_size = 2 if weight_dtype == torch.bfloat16 else 4
+    tile = _train_tile_cols(K, weight_dtype)
+    floor = _hier_min_slice_cols if _hier_min_slice_cols is not None else (64 if tile == 64 else 256)
+    cols = _hier_scratch_budget(B, K, F, D, weight_dtype) // (B * K * p_size)
+    if cols >= tile:
+        cols -= cols % tile  # whole tiles: the library rounds up, the budget is an upper bound
+    return max(floor, cols, 1)
 
 
 def set_hier_scratch_bytes(nbytes) -> None:
-    """Upper bound on the scratch of the hierarchical backward (bytes).  0 = use the atomic
-    scatter fallback, which needs no scratch but an fp32 [F,D] accumulator.  The default (256 MiB)
-    is the size at which one slice of contributions stays in the memory-side cache between the
-    sweep that writes it and the reduction that reads it; wider slices run slower, not faster.
-    ``None`` restores the default."""
+    """Upper bound on the scratch of the hierarchical backward (bytes): the per-pair contributions
+    of one slice of columns.  0 = use the atomic scatter fallback, which needs no scratch but an
+    fp32 [F,D] accumulator.  ``None`` (the default) sizes it from the problem: 0.45 of the weight
+    matrix, at most 256 MiB.  A slice is never narrower than ``set_hier_min_slice_cols``, so with
+    many pairs the scratch can exceed the bound by a large factor (B*K*256 contributions).  Slices
+    of 256 columns measured fastest at B*K = 2^19 pairs; wider ones are not faster."""
     global _hier_scratch_bytes
-    _hier_scratch_bytes = (256 << 20) if nbytes is None else int(nbytes)
+    _hier_scratch_bytes = None if nbytes is None else int(nbytes)
+
+
+# Hot-latent accumulators of the sliced training step (FLEXSAE_BWD_HOT_LATENTS of the library): the
+# most frequent latents of the batch are summed in the LDS by blocks of 128 rows instead of being
+# staged pair by pair.  "auto" takes them where the library supports the shape (16-bit weights,
+# K <= 64) and the batch is sparse in the latents (B*K <= 2F: that is where a few latents in most
+# rows are the usual picture, and where the persistent blocks of that kernel were measured);
+# "on" wherever the shape is supported; "off" never.
+_hot_latents = os.environ.get("FLEXSAE_HOT_LATENTS", "auto").lower()
+_HOT_ROWS_PER_BLOCK = 128  # kHotRowsPerBlock of the library
+
+
+def set_hot_latents(mode) -> None:
+    """``"auto"`` (default), ``"on"``/``True`` or ``"off"``/``False``: whether the sliced hierarchical
+    training step sums the most frequent latents of the batch in LDS accumulators (bit-reproducible
+    fixed-point sums; skewed indices stage about half as many contributions then)."""
+    global _hot_latents
+    if isinstance(mode, bool):
+        mode = "on" if mode else "off"
+    mode = "auto" if mode is None else str(mode).lower()
+    if mode not in ("auto", "on", "off"):
+        raise ValueError("set_hot_latents: expected 'auto', 'on' or 'off'")
+    _hot_latents = mode
+
+
+def _hot_latents_supported(B: int, K: int, F: int, D: int, weight_dtype) -> bool:
+    """flexsae_hier_hot_latents_supported() of the library, restated so that a compiler trace can
+    follow it: 16-bit weights, at most 64 steps, rows the piece reduction can serve."""
+    if weight_dtype not in (torch.bfloat16, torch.float16) or K > 64 or B * K >= 2 ** 31:
+        return False
+    return D % (8 if weight_dtype == torch.bfloat16 else 4) == 0
+
+
+def _use_hot_latents(B: int, K: int, F: int, D: int, weight_dtype) -> bool:
+    if _hot_latents == "off" or not _hot_latents_supported(B, K, F, D, weight_dtype):
+        return False
+    return _hot_latents == "on" or B * K <= 2 * F
+
+
+def _hot_slice_cols(B: int, cols: int, device) -> int:
+    """Slice width for the hot-latent kernel: one block per (128 rows, 128 columns), so a slice
+    should hold a whole number of rounds of one block per compute unit; never narrower than `cols`
+    unless that already is such a width."""
+    n_cu = torch.cuda.get_device_properties(device).multi_processor_count
+    row_blocks = -(-B // _HOT_ROWS_PER_BLOCK)
+    tiles = max(1, round(n_cu / row_blocks))
+    want = 128 * tiles
+    return want if cols <= want else (cols // want) * want
 
 
 # Memory the fused training step may hold between forward and backward: all B*K*D per-pair
@@ -304,9 +379,8 @@ def hier_bwd(grad_out: Tensor, indices: Tensor, weight: Tensor, vals: Tensor,
         shape = _shape(B, K, F, D, weight, vals, torch.float32, torch.float32)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
-        if _hier_scratch_bytes > 0:
-            p_size = 2 if weight.dtype == torch.bfloat16 else 4
-            slice_cols = _hier_slice_cols(B, K, p_size)
+        if _hier_scratch_budget(B, K, F, D, weight.dtype) > 0:
+            slice_cols = _hier_slice_cols(B, K, F, D, weight.dtype)
             ws_bytes = lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
             workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             dW = torch.empty_like(weight)
@@ -443,22 +517,32 @@ def _single_slice_workspace_bytes(lib, shape, D: int) -> int:
     return lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(shape), D)
 
 
-@torch.library.custom_op("flexsae_amd::hier_train", mutates_args=())
-def hier_train(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
-               target: Tensor) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+def hier_train_stage(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, target: Tensor) -> Tensor:
+    """A fresh (uninitialised) stage for ``hier_train``: the workspace that holds the pair list and
+    all per-pair contributions of one step of these shapes.  Eager mode only: the size comes from
+    the library (a host-side query through ctypes, which a compiler trace cannot follow)."""
+    B, K, F, D = _validate(indices, weight, vals, bias, target)
+    shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
+    return torch.empty(_single_slice_workspace_bytes(_lib.load(), shape, D), dtype=torch.uint8, device=weight.device)
+
+
+@torch.library.custom_op("flexsae_amd::hier_train", mutates_args=("stage",))
+def hier_train(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, target: Tensor,
+               stage: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
     """Fused forward + reverse walk with the segment reduction deferred.
 
-    Returns (loss, dvals, dbias, stage): dvals/dbias for a unit upstream gradient, and the
-    workspace holding the pair list and all per-pair contributions, from which
-    ``hier_finish`` produces dW with the upstream gradient folded in."""
+    Returns (loss, dvals, dbias), dvals/dbias for a unit upstream gradient, and fills ``stage``
+    (from ``hier_train_stage``; scratch that the op mutates, not an output: its bytes are of no
+    meaning to the caller and partly unwritten) with the pair list and all per-pair
+    contributions, from which ``hier_finish`` produces dW with the upstream gradient folded in."""
     B, K, F, D = _validate(indices, weight, vals, bias, target)
     lib = _lib.load()
     indices, weight, vals, bias, target = (_prep(t) for t in (indices, weight, vals, bias, target))
     dev = weight.device
+    if stage.dtype != torch.uint8 or stage.device != dev or not stage.is_contiguous():
+        raise ValueError("stage must be a contiguous uint8 tensor on the weight's device (see hier_train_stage)")
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
-        ws_bytes = _single_slice_workspace_bytes(lib, shape, D)
-        stage = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
@@ -469,24 +553,20 @@ def hier_train(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
         flags = _lib.BWD_SWEEP_ONLY | (_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0)
         rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
                                       _ptr(target), _ptr(loss), None, _DTYPES[weight.dtype], _ptr(dvals),
-                                      _ptr(dbias), _ptr(stage), ws_bytes, flags, _ptr(flag), _stream())
-        _lib.check(rc, "flexsae_hier_fwd_bwd")
+                                      _ptr(dbias), _ptr(stage), stage.numel(), flags, _ptr(flag), _stream())
+        _lib.check(rc, "flexsae_hier_fwd_bwd (stage too small or misaligned?)" if rc == _lib.ERR_WORKSPACE
+                   else "flexsae_hier_fwd_bwd")
         if cached is None:
             _pair_export(lib, shape, stage, indices, F)
         if _check_indices:
             check_index_flag(dev)
-    return loss, dvals, dbias, stage
+    return loss, dvals, dbias
 
 
 @hier_train.register_fake
-def _(indices, weight, vals, bias, target):
-    B, K = indices.shape
-    F, D = weight.shape
-    shape = _shape(int(B), int(K), int(F), int(D), weight, vals, bias.dtype, target.dtype)
-    ws_bytes = _single_slice_workspace_bytes(_lib.load(), shape, int(D))  # host-side size query
+def _(indices, weight, vals, bias, target, stage):
     return (weight.new_empty((), dtype=torch.float32), vals.new_empty(vals.shape, dtype=torch.float32),
-            weight.new_empty((weight.shape[1],), dtype=torch.float32),
-            weight.new_empty((ws_bytes,), dtype=torch.uint8))
+            weight.new_empty((weight.shape[1],), dtype=torch.float32))
 
 
 @torch.library.custom_op("flexsae_amd::hier_finish", mutates_args=())
@@ -513,31 +593,32 @@ def _(grad_out, indices, weight, vals, stage):
     return torch.empty_like(weight)
 
 
-def _train_setup_context(ctx, inputs, output):
-    indices, weight, vals, bias, _ = inputs
-    _, dvals, dbias, stage = output
-    ctx.save_for_backward(indices, weight, vals, dvals, dbias, stage)
-    ctx.leaf_dtypes = (vals.dtype, bias.dtype)
-    # unused outputs (the stage above all) must not get zero-filled gradient tensors
-    ctx.set_materialize_grads(False)
+class _HierTrainStaged(torch.autograd.Function):
+    """Autograd glue of the staged step (eager mode): ``hier_train`` fills a fresh stage in the
+    forward, ``hier_finish`` reduces it with the upstream gradient folded in (the counterpart of
+    reference torch-ext/flex_sae/hierarchical_kernels.py:273-299).  ``hier_train`` mutates its stage
+    argument, so it carries no autograd formula of its own."""
 
+    @staticmethod
+    def forward(ctx, indices, weight, vals, bias, target):
+        stage = hier_train_stage(indices, weight, vals, bias, target)
+        loss, dvals, dbias = hier_train(indices, weight, vals, bias, target, stage)
+        ctx.save_for_backward(indices, weight, vals, dvals, dbias, stage)
+        ctx.leaf_dtypes = (vals.dtype, bias.dtype)
+        return loss
 
-def _train_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_stage):
-    indices, weight, vals, dvals, dbias, stage = ctx.saved_tensors
-    if grad_loss is None:
-        return None, None, None, None, None
-    g = grad_loss.to(torch.float32)
-    vdt, bdt = ctx.leaf_dtypes
-    dW = hier_finish(g, indices, weight, vals, stage)
-    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None
-
-
-hier_train.register_autograd(_train_backward, setup_context=_train_setup_context)
+    @staticmethod
+    def backward(ctx, grad_loss):
+        indices, weight, vals, dvals, dbias, stage = ctx.saved_tensors
+        g = grad_loss.to(torch.float32)
+        vdt, bdt = ctx.leaf_dtypes
+        dW = hier_finish(g, indices, weight, vals, stage) if ctx.needs_input_grad[1] else None
+        return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None
 
 
 @torch.library.custom_op("flexsae_amd::hier_train_sliced", mutates_args=())
 def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
-                      target: Tensor, need_dw: bool = True) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+                      target: Tensor, need_dw: bool = True, hot: bool = False) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     """Fused forward + reverse walk in column slices, each reduced right away (flat memory).
 
     Used when the contributions of a whole step do not fit the stage budget: the scratch is one
@@ -551,22 +632,26 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
     dev = weight.device
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
-        p_size = 2 if weight.dtype == torch.bfloat16 else 4
-        slice_cols = _hier_slice_cols(B, K, p_size)
-        ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
+        slice_cols = _hier_slice_cols(B, K, F, D, weight.dtype)
+        hot_flag = _lib.BWD_HOT_LATENTS if (hot and need_dw) else 0
+        if hot_flag:
+            slice_cols = _hot_slice_cols(B, slice_cols, dev)
+        ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(shape), slice_cols, hot_flag)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
-        dW = torch.empty_like(weight) if need_dw else weight.new_empty((0, D))
+        dw_dtype = _unit_dw_dtype(weight.dtype)
+        dW = torch.empty((F, D), dtype=dw_dtype, device=dev) if need_dw else weight.new_empty((0, D), dtype=dw_dtype)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
         dbias = torch.empty((D,), dtype=torch.float32, device=dev)
         flag = _flag_for(dev)
         cached = _pair_lookup(indices, F)
         if cached is not None:
             _pair_import(lib, shape, workspace, cached)
-        flags = (_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0) | (0 if need_dw else _lib.BWD_NO_DW)
+        flags = ((_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0) | (0 if need_dw else _lib.BWD_NO_DW) |
+                 hot_flag)
         rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
                                       _ptr(target), _ptr(loss), _ptr(dW) if need_dw else None,
-                                      _DTYPES[weight.dtype], _ptr(dvals),
+                                      _DTYPES[dw_dtype], _ptr(dvals),
                                       _ptr(dbias), _ptr(workspace), ws_bytes, flags, _ptr(flag), _stream())
         _lib.check(rc, "flexsae_hier_fwd_bwd")
         if cached is None:
@@ -576,11 +661,18 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
     return loss, dvals, dbias, dW
 
 
+def _unit_dw_dtype(weight_dtype):
+    """dtype of the unit-gradient dW of the sliced step: the weight's, but fp32 for fp16 weights."""
+    return torch.float32 if weight_dtype == torch.float16 else weight_dtype
+
+
 @hier_train_sliced.register_fake
-def _(indices, weight, vals, bias, target, need_dw=True):
+def _(indices, weight, vals, bias, target, need_dw=True, hot=False):
+    dw_dtype = _unit_dw_dtype(weight.dtype)
     return (weight.new_empty((), dtype=torch.float32), vals.new_empty(vals.shape, dtype=torch.float32),
             weight.new_empty((weight.shape[1],), dtype=torch.float32),
-            torch.empty_like(weight) if need_dw else weight.new_empty((0, weight.shape[1])))
+            weight.new_empty(weight.shape, dtype=dw_dtype) if need_dw
+            else weight.new_empty((0, weight.shape[1]), dtype=dw_dtype))
 
 
 @torch.library.custom_op("flexsae_amd::hier_sgd_step", mutates_args=("weight",))
@@ -609,8 +701,7 @@ def hier_sgd_step(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, t
     dev = weight.device
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
-        p_size = 2 if weight.dtype == torch.bfloat16 else 4
-        slice_cols = _hier_slice_cols(B, K, p_size)
+        slice_cols = _hier_slice_cols(B, K, F, D, weight.dtype)
         ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
@@ -672,6 +763,29 @@ def _(x, grad_out):
     return torch.empty_like(x)
 
 
+@torch.library.custom_op("flexsae_amd::scale_to", mutates_args=())
+def scale_to(x: Tensor, grad_out: Tensor, dtype: torch.dtype) -> Tensor:
+    """(x * grad_out) rounded once to ``dtype``; x is fp32.  For fp16 weights: the unit-gradient dW is
+    kept in fp32 and takes the upstream gradient (a loss scale, typically) before it is rounded, like
+    the reference's fp32 ``mul_`` followed by the engine's cast (hierarchical_kernels.py:294-299)."""
+    if x.dtype != torch.float32:
+        raise TypeError("scale_to expects a float32 tensor")
+    lib = _lib.load()
+    dev = x.device
+    with torch.cuda.device(dev):
+        g = _grad_scalar(grad_out, dev)
+        x = _prep(x)
+        out = torch.empty(x.shape, dtype=dtype, device=dev)
+        rc = lib.flexsae_scale_from_f32(_ptr(out), _DTYPES[dtype], _ptr(x), x.numel(), _ptr(g), _stream())
+        _lib.check(rc, "flexsae_scale_from_f32")
+    return out
+
+
+@scale_to.register_fake
+def _(x, grad_out, dtype):
+    return x.new_empty(x.shape, dtype=dtype)
+
+
 @torch.library.custom_op("flexsae_amd::scale_", mutates_args=("x",))
 def scale_(x: Tensor, grad_out: Tensor) -> None:
     """x *= grad_out in place (x contiguous); a grad_out of exactly one costs an empty launch."""
@@ -696,8 +810,9 @@ def _is_traced(t: Tensor) -> bool:
 
 
 def _train_sliced_setup_context(ctx, inputs, output):
-    indices, weight, vals, bias, target, need_dw = inputs
+    indices, weight, vals, bias, target, need_dw, hot = inputs
     ctx.need_dw = need_dw
+    ctx.hot = hot
     _, dvals, dbias, dW = output
     ctx.mark_non_differentiable(dvals, dbias, dW)
     ctx.leaf_dtypes = (vals.dtype, bias.dtype)
@@ -715,14 +830,16 @@ def _train_sliced_setup_context(ctx, inputs, output):
 
 def _train_sliced_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_dw):
     if grad_loss is None:
-        return None, None, None, None, None, None
+        return None, None, None, None, None, None, None
     if ctx.needs_input_grad[1] and not ctx.need_dw:
         raise RuntimeError("hier_train_sliced was called with need_dw=False but weight requires a gradient")
     g = grad_loss.to(torch.float32)
     vdt, bdt = ctx.leaf_dtypes
     if not ctx.dw_in_place:
         indices, weight, vals, bias, target, dvals, dbias, dW_unit = ctx.saved_tensors
-        dW = scale_by(dW_unit, g) if ctx.needs_input_grad[1] else None
+        dW = None
+        if ctx.needs_input_grad[1]:
+            dW = scale_by(dW_unit, g) if dW_unit.dtype == weight.dtype else scale_to(dW_unit, g, weight.dtype)
     else:
         indices, weight, vals, bias, target, dvals, dbias = ctx.saved_tensors
         dW = None
@@ -732,9 +849,12 @@ def _train_sliced_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_dw):
             if dW is None:
                 # a second backward through a retained graph: the buffer went with the first one
                 with torch.no_grad():
-                    _, dvals, dbias, dW = hier_train_sliced(indices, weight, vals, bias, target)
-            scale_(dW, g)
-    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None, None
+                    _, dvals, dbias, dW = hier_train_sliced(indices, weight, vals, bias, target, True, ctx.hot)
+            if dW.dtype == weight.dtype:
+                scale_(dW, g)
+            else:  # fp16 weights: the fp32 unit gradient meets the upstream gradient before its only rounding
+                dW = scale_to(dW, g, weight.dtype)
+    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None, None, None
 
 
 hier_train_sliced.register_autograd(_train_sliced_backward, setup_context=_train_sliced_setup_context)
@@ -779,15 +899,17 @@ def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, 
     needs_grad = torch.is_grad_enabled() and (weight.requires_grad or vals.requires_grad or bias.requires_grad)
     if (needs_grad and _fused_training and weight.dim() == 2 and indices.dim() == 2
             and _train_supported(weight, indices.shape[1])):
-        if _stage_fits(indices, weight):
-            return hier_train(indices, weight, vals, bias, target)[0]
-        # The slice-by-slice step rounds the unit-gradient dW to the weight dtype before the backward
-        # scales it.  fp16 cannot hold gradients of magnitude 2/(B*K*D) (they would be flushed before
-        # a loss-scaling grad_out lifts them), so fp16 weights take the separate forward + backward,
-        # which folds grad_out in before the only rounding (reference hierarchical_kernels.py:294-299
-        # scales in fp32 as well).
-        if _hier_scratch_bytes > 0 and not (weight.requires_grad and weight.dtype == torch.float16):
-            return hier_train_sliced(indices, weight, vals, bias, target, bool(weight.requires_grad))[0]
+        # (a compiler trace cannot follow the stage's size query: traced calls take the sliced step,
+        # which gives the same bits)
+        if _stage_fits(indices, weight) and not _is_traced(weight):
+            return _HierTrainStaged.apply(indices, weight, vals, bias, target)
+        # (fp16 weights: the step's unit-gradient dW is fp32, of magnitude 2/(B*K*D), and is scaled by the
+        # upstream gradient before its only rounding, like reference hierarchical_kernels.py:294-299)
+        if _hier_scratch_bytes != 0:
+            B, K = indices.shape
+            F, D = weight.shape
+            hot = bool(weight.requires_grad) and _use_hot_latents(B, K, F, D, weight.dtype)
+            return hier_train_sliced(indices, weight, vals, bias, target, bool(weight.requires_grad), hot)[0]
     return hier_fwd(indices, weight, vals, bias, target)[0]
 
 

@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define FLEXSAE_ABI_VERSION 2
+#define FLEXSAE_ABI_VERSION 3
 
 typedef enum {
   FLEXSAE_OK = 0,
@@ -73,10 +73,26 @@ enum {
   FLEXSAE_TOPK_BWD_FP32_RESIDUAL = 256, /* flexsae_topk_bwd with bf16 weights: gather the fp32  */
                                      /* residual instead of a bf16 copy of it (slower, and dvals */
                                      /* then carry fp32 rounding only instead of bf16's)         */
-  FLEXSAE_BWD_SKIP_EPILOGUE = 64     /* measurement aid for flexsae_hier_fwd_bwd: leave out the */
-                                     /* kernels that finish loss, dvals and dbias (those        */
-                                     /* outputs are then not written), so that a call with      */
-                                     /* NO_DW or SWEEP_ONLY runs the training-step kernel alone */
+  FLEXSAE_BWD_HOT_LATENTS = 128,     /* flexsae_hier_fwd_bwd / flexsae_hier_sgd_step: give the  */
+                                     /* most frequent latents of the batch accumulators in the  */
+                                     /* LDS (see flexsae_hier_hot_latents_supported); a hint,   */
+                                     /* ignored where the shape or the call does not allow it.  */
+                                     /* The workspace must come from                            */
+                                     /* flexsae_hier_fwd_bwd_workspace_bytes_flags(.., flags)   */
+  FLEXSAE_BWD_REUSE_HOT_TABLES = 1024, /* with REUSE_PAIR_LIST and HOT_LATENTS: the workspace   */
+                                     /* also still holds the hot-latent tables of a previous    */
+                                     /* call with HOT_LATENTS on the same indices and shape     */
+  FLEXSAE_BWD_HOT_NO_HEADROOM = 512, /* NOT PART OF THE STABLE ABI (a test aid): the block      */
+                                     /* exponent of the hot-latent accumulators is set 8 bits   */
+                                     /* lower than usual, so that most rows take the deferred   */
+                                     /* second pass; results stay valid                         */
+  FLEXSAE_BWD_SKIP_EPILOGUE = 64     /* NOT PART OF THE STABLE ABI (a measurement aid of this   */
+                                     /* library's own benchmark, with no counterpart in the     */
+                                     /* reference; may change or go without an ABI bump).       */
+                                     /* flexsae_hier_fwd_bwd: leave out the kernels that finish */
+                                     /* loss, dvals and dbias (those outputs are then not       */
+                                     /* written), so that a call with NO_DW or SWEEP_ONLY runs  */
+                                     /* the training-step kernel alone                          */
 };
 
 /* Problem description.  Limits: 1 <= B,K,F,D; F < 2^31; D < 2^29; B*K < 2^32. */
@@ -198,10 +214,37 @@ int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const v
  * and to whole 256-column tiles otherwise; slice_cols <= 0 asks for the minimum; 0 is returned for
  * unsupported shapes.  Narrow slices keep one slice of contributions in the memory-side cache
  * between the kernel that writes it and the reduction that reads it.  A workspace from
- * flexsae_hier_bwd_workspace_bytes is accepted as well.
+ * flexsae_hier_bwd_workspace_bytes is accepted as well.  The query assumes a dW aligned for that
+ * 16-byte lane width (4 elements of fp32 or fp16 contributions' gradient, 8 of bf16); a dW aligned
+ * less than that switches the piece reduction off, slices are then whole 256-column tiles, and a
+ * workspace of the minimum width from this query is answered with FLEXSAE_ERR_WORKSPACE: ask
+ * flexsae_hier_bwd_workspace_bytes instead.
  */
 int flexsae_hier_fwd_bwd_supported(const flexsae_shape *shape);
 size_t flexsae_hier_fwd_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slice_cols);
+/*
+ * Hot-latent accumulators (FLEXSAE_BWD_HOT_LATENTS): where indices are skewed, a few latents are
+ * selected by most batch rows, and the reference's backward piles its atomic adds up on their rows
+ * of dW (hierarchical_kernels.py:155-161).  With the flag, the (up to 288) latents with the most
+ * pairs -- more than 64 and no batch row holding the latent twice -- are summed in LDS accumulators
+ * by blocks of 128 batch rows instead of being staged pair by pair, in 32-bit fixed point with one
+ * exponent per block (integer sums do not depend on the order of the additions: results stay
+ * bit-reproducible, and identical for every slice width).  Supported for 16-bit weights with
+ * K <= 64 and D a multiple of 8 (bf16) or 4 (fp16); `_supported` says whether the flag would be
+ * honoured for `shape`, `_workspace_bytes_flags` is the workspace query for a call with `flags`
+ * (the accumulators' block partials take (slice columns / 128) x ceil(B / 128) x 147456 bytes, twice).
+ * Slices are best chosen so that (slice columns / 128) x ceil(B / 128) is a multiple of the number
+ * of compute units (one block each).
+ */
+int flexsae_hier_hot_latents_supported(const flexsae_shape *shape);
+size_t flexsae_hier_fwd_bwd_workspace_bytes_flags(const flexsae_shape *shape, int64_t slice_cols, int flags);
+/*
+ * What the last call with FLEXSAE_BWD_HOT_LATENTS on `workspace` did (a diagnostic with no counterpart
+ * in the reference): stats[0..5) (device memory) = hot latents, candidates (latents above the pair-count
+ * threshold), long latents left to the chunked reduction, the threshold, and the number of
+ * (row, tile) walks that were deferred to the second pass, summed over the slices.
+ */
+int flexsae_hier_hot_stats(const flexsae_shape *shape, const void *workspace, uint32_t *stats, void *stream);
 int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
                          const void *vals, const void *bias, const void *target, float *loss,
                          void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,
@@ -218,8 +261,10 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, con
  * dvals is what the encoder's backward needs, dbias the bias's update) and are computed from the
  * weights as they were on entry: within a slice of columns every read of the weights precedes the
  * reduction that updates that slice, and other slices touch other columns.
- * Supported where flexsae_hier_fwd_bwd is and D is a multiple of 8 (16-bit weights) or 4 (fp32)
- * with a 16-byte aligned weight matrix; otherwise FLEXSAE_ERR_UNSUPPORTED.  Workspace as for
+ * Supported where flexsae_hier_fwd_bwd is and the reduction can work 16 bytes per lane on the
+ * staged contributions: D a multiple of 8 for bf16 weights (bf16 contributions, weight rows 16-byte
+ * aligned), of 4 for fp32 and fp16 weights (fp32 contributions; weight rows aligned to 4 elements:
+ * 16 bytes for fp32, 8 for fp16); otherwise FLEXSAE_ERR_UNSUPPORTED.  Workspace as for
  * flexsae_hier_fwd_bwd; the only flag accepted is FLEXSAE_BWD_REUSE_PAIR_LIST.
  * replaces: the dense dW of the backward (hierarchical_kernels.py:241-243, 294-297) together with
  *           the optimizer pass that consumes it in a training loop written like reference
@@ -312,8 +357,9 @@ int flexsae_topk_bwd(const flexsae_shape *shape, const uint32_t *begin, const ui
  * (rounded to whole tiles, capped at D; <= 0 asks for the minimum).  The slice width only
  * sizes the fp32 partial sums of latents with more than 64 pairs (hot latents are cut into
  * 64-pair chunks that are reduced by separate wavefronts and then combined in a fixed order);
- * the fixed part holds the per-pair records, the per-tile dvals shares (D/256 x B*K fp32) and,
- * for bf16 weights, the bf16 residual copy.
+ * the fixed part holds the per-pair records, the per-tile dvals shares (one fp32 per pair and
+ * tile) and, for bf16 weights, the bf16 residual copy.  The result covers both layouts of the
+ * call, with and without FLEXSAE_TOPK_BWD_FP32_RESIDUAL (the larger of the two).
  */
 size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slice_cols);
 
@@ -324,6 +370,17 @@ size_t flexsae_topk_bwd_workspace_bytes(const flexsae_shape *shape, int64_t slic
  *           hierarchical_kernels.py:299.
  */
 int flexsae_cast_from_f32(void *dst, int dst_dtype, const float *src, int64_t n, void *stream);
+
+/*
+ * dst[n] (dtype) = src[n] (fp32) * scale[0], one rounding (`scale` a device fp32 scalar; NULL = 1).
+ * For gradients of fp16 weights: the unit-gradient dW of flexsae_hier_fwd_bwd is of magnitude
+ * 2/(B*K*D), below fp16's range, so it is kept in fp32 and meets the upstream gradient (a loss
+ * scale, typically) before the only rounding.
+ * replaces: dW.mul_(grad) in fp32 followed by the engine's cast to the leaf dtype
+ *           (hierarchical_kernels.py:294-299).
+ */
+int flexsae_scale_from_f32(void *dst, int dst_dtype, const float *src, int64_t n, const float *scale,
+                           void *stream);
 
 #ifdef __cplusplus
 }

@@ -59,9 +59,10 @@ def hier_backward(indices, weight, vals, resid, grad_out, flag=None, slice_cols=
 
 
 def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_dtype=torch.float32, flags=0,
-               alloc_dw=True):
+               alloc_dw=True, keep_workspace=False):
     """Fused forward+backward for a unit upstream gradient -> (rc, loss, dW, dvals, dbias);
-    ``alloc_dw=False`` passes a null dW (for FLEXSAE_BWD_NO_DW)."""
+    ``alloc_dw=False`` passes a null dW (for FLEXSAE_BWD_NO_DW); ``keep_workspace`` appends the
+    workspace to the result (for flexsae_hier_hot_stats)."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
     dev = weight.device
@@ -70,16 +71,28 @@ def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_
     dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
     db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
     # slices of whole training tiles where the entry point supports the shape
-    nbytes = (lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+    nbytes = (lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(sh), slice_cols, flags)
               or lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols))
     ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
     rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(bias), ptr(target),
                                   ptr(loss), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, flags,
                                   ptr(flag), stream())
+    if keep_workspace:
+        return rc, loss, dW, dv, db, ws
     return rc, loss, dW, dv, db
 
 
-def hier_sgd_step(indices, weight, vals, bias, target, step, flag=None, slice_cols=0):
+def hot_stats(indices, weight, vals, bias, target, workspace):
+    """flexsae_hier_hot_stats -> [hot latents, candidates, cold long latents, threshold, deferred walks]."""
+    lib = _lib.load()
+    sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
+    stats = torch.zeros(5, dtype=torch.int32, device=weight.device)
+    rc = lib.flexsae_hier_hot_stats(ctypes.byref(sh), ptr(workspace), ptr(stats), stream())
+    assert rc == 0, _lib.status_string(rc)
+    return [int(x) for x in stats.cpu()]
+
+
+def hier_sgd_step(indices, weight, vals, bias, target, step, flag=None, slice_cols=0, flags=0):
     """Training step with the SGD update of ``weight`` fused in (in place) -> (rc, loss, dvals, dbias)."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
@@ -87,11 +100,11 @@ def hier_sgd_step(indices, weight, vals, bias, target, step, flag=None, slice_co
     loss = torch.full((1,), float("nan"), dtype=torch.float32, device=dev)
     dv = torch.full((sh.B, sh.K), float("nan"), dtype=torch.float32, device=dev)
     db = torch.full((sh.D,), float("nan"), dtype=torch.float32, device=dev)
-    nbytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(sh), slice_cols)
+    nbytes = lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(sh), slice_cols, flags)
     ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
     st = torch.tensor([step], dtype=torch.float32, device=dev)
     rc = lib.flexsae_hier_sgd_step(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(bias), ptr(target),
-                                   ptr(st), ptr(loss), ptr(dv), ptr(db), ptr(ws), nbytes, 0, ptr(flag), stream())
+                                   ptr(st), ptr(loss), ptr(dv), ptr(db), ptr(ws), nbytes, flags, ptr(flag), stream())
     return rc, loss, dv, db
 
 

@@ -1,0 +1,137 @@
+"""Hot-latent accumulators of the training step (FLEXSAE_BWD_HOT_LATENTS), through the C ABI.
+
+The most frequent latents of a batch are summed in LDS accumulators (32-bit fixed point, one
+exponent per block of 128 rows) instead of being staged pair by pair.  Checked here: parity with the
+oracle on skewed indices (every K variant of the kernel, bf16 and fp16 weights, a ragged last row
+block, more long latents than accumulator rows), that loss / dvals / dbias are the bits of the plain
+step, that latents with a repeated row stay cold (duplicates: dW bit-identical to the plain step),
+the deferred second pass (forced by FLEXSAE_BWD_HOT_NO_HEADROOM), bit-identical dW for every slice
+width and from run to run, and the fused SGD update.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import abi
+from flexsae_amd import _lib
+import oracle
+from helpers import make_inputs, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+HOT = _lib.BWD_HOT_LATENTS
+
+
+def _dev(args):
+    return tuple(x.to(DEV) for x in args)
+
+
+def _supported(idx, W, v, b, t):
+    sh = abi.shape_of(idx, W, v, b.dtype, t.dtype)
+    return bool(_lib.load().flexsae_hier_hot_latents_supported(ctypes.byref(sh)))
+
+
+def _check_vs_oracle(cpu_args, dW, dv, db, loss, tol):
+    L, rW, rv, rb = oracle.loss_grads(oracle.HIER, *cpu_args)
+    assert abs(loss.item() - L) <= max(tol * 1e-1, 1e-5) * abs(L)
+    assert rel_err(dv.cpu(), rv) <= tol
+    assert rel_err(db.cpu(), rb) <= tol
+    got, ref = dW.double().cpu(), torch.from_numpy(rW)
+    assert rel_err(got, ref) <= tol
+    # element by element too: |got - ref| <= tol |ref| + tol max|ref|
+    assert float(((got - ref).abs() - tol * ref.abs()).max()) <= tol * float(ref.abs().max())
+    return ref
+
+
+@pytest.mark.parametrize("shape,dtype,zipf", [
+    ((300, 64, 2000, 512), torch.bfloat16, 1.1),     # ragged last row block, full 64-step kernel
+    ((256, 32, 1500, 264), torch.bfloat16, 1.2),     # 32 steps, D not a whole tile
+    ((200, 16, 900, 128), torch.bfloat16, 1.3),      # 16 steps
+    ((260, 40, 1200, 384), torch.bfloat16, 1.1),     # K below the kernel's bound (per-step tests)
+    ((384, 64, 1800, 256), torch.float16, 1.1),      # fp16 weights: fp32 contributions, fp32 dW
+    ((2048, 64, 1000, 128), torch.bfloat16, 0.3),    # more long latents than accumulator rows
+])
+def test_hot_latents_match_the_oracle(shape, dtype, zipf):
+    print("[case] hot", shape, dtype, zipf, flush=True)
+    cpu_args = make_inputs(*shape, dtype, seed=31, zipf_s=zipf, sort_vals=True, w_std=0.3)
+    args = _dev(cpu_args)
+    assert _supported(*args)
+    dw_dtype = torch.float32 if dtype == torch.float16 else dtype
+    rc0, loss0, dW0, dv0, db0 = abi.hier_train(*args, dw_dtype=dw_dtype, slice_cols=256)
+    rc, loss, dW, dv, db, ws = abi.hier_train(*args, dw_dtype=dw_dtype, slice_cols=256, flags=HOT, keep_workspace=True)
+    assert rc0 == 0 and rc == 0, (_lib.status_string(rc0), _lib.status_string(rc))
+    n_hot, n_cand, n_cold_long, threshold, deferred = abi.hot_stats(*args, ws)
+    counts = np.bincount(cpu_args[0].numpy().ravel(), minlength=shape[2])
+    n_long = int((counts > 64).sum())
+    assert n_hot == n_cand == min(n_long, int((counts > threshold).sum())) and 0 < n_hot <= 288  # per-row unique indices
+    assert n_cold_long == n_long - n_hot and deferred == 0
+    if n_long > 288:  # the threshold is the 289th largest pair count
+        assert threshold == int(np.sort(counts)[-289])
+    # the hot latents change nothing but dW
+    assert torch.equal(loss, loss0) and torch.equal(dv, dv0) and torch.equal(db, db0)
+    assert n_long > 0, "the case has no frequent latent"
+    assert not torch.equal(dW, dW0), "the hot path was not taken"
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-4
+    ref = _check_vs_oracle(cpu_args, dW, dv, db, loss, tol)
+    # rows of the frequent latents: fixed point with 23 bits below the block's bound is far more
+    # exact than one bf16 rounding per contribution
+    hot_rows = torch.from_numpy(np.argsort(-counts)[:16].copy())
+    e_hot = rel_err(dW[hot_rows.to(DEV)].double().cpu(), ref[hot_rows])
+    e_plain = rel_err(dW0[hot_rows.to(DEV)].double().cpu(), ref[hot_rows])
+    assert e_hot <= (4e-3 if dtype == torch.bfloat16 else 2e-5), (e_hot, e_plain)
+
+
+def test_repeated_rows_keep_a_latent_cold():
+    """randint indices on few latents: every latent is frequent and nearly every one is repeated
+    inside some row, so none may be summed in the accumulators: dW is the plain step's, bit for bit."""
+    print("[case] hot duplicates", flush=True)
+    args = _dev(make_inputs(192, 64, 96, 256, torch.bfloat16, seed=5))
+    rc0, _, dW0, _, _ = abi.hier_train(*args, dw_dtype=torch.bfloat16)
+    rc, _, dW, _, _ = abi.hier_train(*args, dw_dtype=torch.bfloat16, flags=HOT)
+    assert rc0 == 0 and rc == 0
+    assert torch.equal(dW, dW0)
+
+
+def test_deferred_rows_and_reproducibility():
+    """With the block exponent set 8 bits low most rows exceed it, are left out of the first pass
+    and walked again after the exponent has been raised: still the oracle's dW, the same bits on
+    every run and for every slice width; and so for the normal headroom."""
+    print("[case] hot deferred", flush=True)
+    cpu_args = make_inputs(300, 64, 2000, 512, torch.bfloat16, seed=32, zipf_s=1.1, sort_vals=True, w_std=0.3)
+    # rows of very different magnitude: the later rows of every block dwarf its first ones
+    scale = torch.ones(300)
+    scale[40::3] = 64.0
+    cpu_args = (cpu_args[0], cpu_args[1], cpu_args[2], cpu_args[3], (cpu_args[4].float() * scale[:, None]).to(torch.bfloat16))
+    args = _dev(cpu_args)
+    for extra in (0, _lib.BWD_HOT_NO_HEADROOM):
+        outs = []
+        for cols in (128, 256, 512, 128):
+            rc, loss, dW, dv, db, ws = abi.hier_train(*args, dw_dtype=torch.bfloat16, slice_cols=cols, flags=HOT | extra,
+                                                      keep_workspace=True)
+            assert rc == 0
+            deferred = abi.hot_stats(*args, ws)[4]
+            print("deferred walks", deferred, "of", 300 * 4, flush=True)
+            assert deferred > (300 if extra else 0)
+            outs.append(dW)
+        for o in outs[1:]:
+            assert torch.equal(o, outs[0])
+        _check_vs_oracle(cpu_args, outs[0], dv, db, loss, 1e-2)
+
+
+def test_sgd_update_with_hot_latents():
+    print("[case] hot sgd", flush=True)
+    cpu_args = make_inputs(300, 64, 2000, 512, torch.bfloat16, seed=33, zipf_s=1.1, sort_vals=True, w_std=0.3)
+    idx, W, v, b, t = _dev(cpu_args)
+    step = 0.37
+    Wn = W.clone()
+    rc, loss, dv, db = abi.hier_sgd_step(idx, Wn, v, b, t, step, slice_cols=256, flags=HOT)
+    assert rc == 0, _lib.status_string(rc)
+    L, rW, rv, rb = oracle.loss_grads(oracle.HIER, *cpu_args)
+    want = cpu_args[1].double() - step * torch.from_numpy(rW)
+    touched = torch.from_numpy(np.bincount(cpu_args[0].numpy().ravel(), minlength=2000) > 0)
+    # update = step * dW: compare the change, within bf16's rounding of the new weights
+    assert rel_err(Wn.double().cpu()[touched], want[touched]) <= 4e-3
+    assert torch.equal(Wn.cpu()[~touched], cpu_args[1][~touched])
+    assert abs(loss.item() - L) <= 1e-3 * abs(L) and rel_err(dv.cpu(), rv) <= 1e-2
