@@ -309,7 +309,7 @@ def main():
     hier_mode = "staged" if staged else "sliced" if fused else "unfused"
     slice_cols = D if staged else flex.ops._hier_slice_cols(B, K, F, D, dtype)
     # hot-latent accumulators: the same decision as the API takes for a weight that needs its gradient
-    hot = bool(fused and not staged and flex.ops._use_hot_latents(B, K, F, D, dtype))
+    hot = bool(fused and not staged and flex.ops._use_hot_latents(B, K, F, D, dtype, dev))
     HOTF = _lib.BWD_HOT_LATENTS if hot else 0
     if hot:
         slice_cols = flex.ops._hot_slice_cols(B, slice_cols, dev)

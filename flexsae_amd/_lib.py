@@ -86,6 +86,7 @@ SIGNATURES = {
     "flexsae_scale_from_f32": (_int, [_p, _int, _p, _i64, _p, _p]),
     "flexsae_hier_hot_latents_supported": (_int, [_shape_p]),
     "flexsae_hier_hot_stats": (_int, [_shape_p, _p, _p, _p]),
+    "flexsae_hier_pair_stats": (_int, [_shape_p, _p, _p, _p]),
     "flexsae_hier_fwd_bwd_workspace_bytes_flags": (_sz, [_shape_p, _i64, _int]),
 }
 

@@ -1188,6 +1188,19 @@ int flexsae_hier_hot_latents_supported(const flexsae_shape *s) {
   return check_shape(s) == FLEXSAE_OK && train_supported(s) && hot_supported(s) ? 1 : 0;
 }
 
+int flexsae_hier_pair_stats(const flexsae_shape *s, const void *workspace, uint32_t *stats, void *stream) {
+  const int rc = check_shape(s);
+  if (rc != FLEXSAE_OK) return rc;
+  if (!workspace || !stats) return FLEXSAE_ERR_INVALID_ARGUMENT;
+  if (!aligned(workspace, kAlign) || !aligned(stats, 4)) return FLEXSAE_ERR_ALIGNMENT;
+  const HierBwdPlan pl = plan_hier_bwd(s);  // the part of the layout every hierarchical workspace shares
+  uint8_t *ws = static_cast<uint8_t *>(const_cast<void *>(workspace));
+  const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
+  hipLaunchKernelGGL(pair_stats_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), sc.long_count,
+                     reinterpret_cast<const uint32_t *>(ws + pl.off_chunk), stats);
+  return launch_status();
+}
+
 int flexsae_hier_hot_stats(const flexsae_shape *s, const void *workspace, uint32_t *stats, void *stream) {
   const int rc = check_shape(s);
   if (rc != FLEXSAE_OK) return rc;

@@ -198,6 +198,17 @@ __global__ void hot_cold_long_kernel(const uint32_t *__restrict__ long_count,
   }
 }
 
+// out[0] = latents with more than kSegChunk pairs, out[1] = their 64-pair chunks (so between
+// out[1] * 64 - 63 * out[0] and out[1] * 64 pairs belong to them).  `out` may be pinned host memory.
+__global__ void pair_stats_kernel(const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ chunk_begin,
+                                  uint32_t *__restrict__ out) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    const uint32_t n_long = *long_count;
+    out[0] = n_long;
+    out[1] = chunk_begin[n_long];
+  }
+}
+
 // ---- second step of the hot latents ---------------------------------------------------------
 // out[f, tile] = sum over the row blocks of the block partials of hot latent f, in block order
 // (four running sums, combined as (s0 + s1) + (s2 + s3)).  The partials keep the accumulators'

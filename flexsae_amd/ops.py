@@ -237,18 +237,25 @@ def set_hier_scratch_bytes(nbytes) -> None:
 
 # Hot-latent accumulators of the sliced training step (FLEXSAE_BWD_HOT_LATENTS of the library): the
 # most frequent latents of the batch are summed in the LDS by blocks of 128 rows instead of being
-# staged pair by pair.  "auto" takes them where the library supports the shape (16-bit weights,
-# K <= 64) and the batch is sparse in the latents (B*K <= 2F: that is where a few latents in most
-# rows are the usual picture, and where the persistent blocks of that kernel were measured);
-# "on" wherever the shape is supported; "off" never.
+# staged pair by pair.  That pays where indices are skewed (a few latents in most rows) and costs
+# where they are not (its blocks hold the LDS of a whole compute unit: half the wavefronts of the
+# plain kernel), and only the device knows which it is.  "auto" therefore measures: every sliced step
+# leaves, in pinned host memory, how many of its pairs belong to latents with more than 64 pairs
+# (flexsae_hier_pair_stats; no synchronisation: an event is polled), and the next step of the same
+# shape on the same device takes the accumulators when that was a quarter of the pairs or more.  The
+# first step of a shape, and steps traced by a compiler, run the plain kernel.
+# "on" takes them wherever the shape is supported (16-bit weights, K <= 64); "off" never.
 _hot_latents = os.environ.get("FLEXSAE_HOT_LATENTS", "auto").lower()
-_HOT_ROWS_PER_BLOCK = 128  # kHotRowsPerBlock of the library
+_HOT_ROWS_PER_BLOCK = 128   # kHotRowsPerBlock of the library
+_HOT_AUTO_FRACTION = 0.25   # of the pairs in latents with more than 64 pairs
+_hot_auto = {}              # (device index, B, K, F, D, dtype) -> {"hot", "pinned", "event"}
 
 
 def set_hot_latents(mode) -> None:
     """``"auto"`` (default), ``"on"``/``True`` or ``"off"``/``False``: whether the sliced hierarchical
     training step sums the most frequent latents of the batch in LDS accumulators (bit-reproducible
-    fixed-point sums; skewed indices stage about half as many contributions then)."""
+    fixed-point sums; skewed indices stage about half as many contributions then).  ``"auto"``
+    decides from the previous step of the same shape (see the module's comment)."""
     global _hot_latents
     if isinstance(mode, bool):
         mode = "on" if mode else "off"
@@ -256,6 +263,7 @@ def set_hot_latents(mode) -> None:
     if mode not in ("auto", "on", "off"):
         raise ValueError("set_hot_latents: expected 'auto', 'on' or 'off'")
     _hot_latents = mode
+    _hot_auto.clear()
 
 
 def _hot_latents_supported(B: int, K: int, F: int, D: int, weight_dtype) -> bool:
@@ -266,10 +274,44 @@ def _hot_latents_supported(B: int, K: int, F: int, D: int, weight_dtype) -> bool
     return D % (8 if weight_dtype == torch.bfloat16 else 4) == 0
 
 
-def _use_hot_latents(B: int, K: int, F: int, D: int, weight_dtype) -> bool:
+def _hot_key(device, B, K, F, D, weight_dtype):
+    return (device.index if device.index is not None else torch.cuda.current_device(), B, K, F, D, weight_dtype)
+
+
+def _use_hot_latents(B: int, K: int, F: int, D: int, weight_dtype, device=None, traced: bool = False) -> bool:
     if _hot_latents == "off" or not _hot_latents_supported(B, K, F, D, weight_dtype):
         return False
-    return _hot_latents == "on" or B * K <= 2 * F
+    if _hot_latents == "on":
+        return True
+    if traced or device is None or torch.cuda.is_current_stream_capturing():
+        return False  # (a graph under capture keeps whatever kernel it captured)
+    st = _hot_auto.get(_hot_key(device, B, K, F, D, weight_dtype))
+    if st is None:
+        return False
+    if st["event"] is not None and st["event"].query():  # the previous step's measurement has arrived
+        long_pairs = int(st["pinned"][1]) * 64
+        st["hot"] = long_pairs >= _HOT_AUTO_FRACTION * B * K
+        st["event"] = None
+    return st["hot"]
+
+
+def _hot_measure(lib, shape, workspace: Tensor, B, K, F, D, weight_dtype) -> None:
+    """Leave the skew of this step's indices where the next step of the shape finds it."""
+    if _hot_latents != "auto" or not _hot_latents_supported(B, K, F, D, weight_dtype):
+        return
+    if torch.cuda.is_current_stream_capturing():
+        return
+    key = _hot_key(workspace.device, B, K, F, D, weight_dtype)
+    st = _hot_auto.get(key)
+    if st is None:
+        st = _hot_auto[key] = {"hot": False, "pinned": torch.zeros(2, dtype=torch.int32, pin_memory=True), "event": None}
+    if st["event"] is not None:
+        return  # a measurement is still on its way
+    rc = lib.flexsae_hier_pair_stats(ctypes.byref(shape), _ptr(workspace), _ptr(st["pinned"]), _stream())
+    _lib.check(rc, "flexsae_hier_pair_stats")
+    ev = torch.cuda.Event()
+    ev.record()
+    st["event"] = ev
 
 
 def _hot_slice_cols(B: int, cols: int, device) -> int:
@@ -656,6 +698,8 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
         _lib.check(rc, "flexsae_hier_fwd_bwd")
         if cached is None:
             _pair_export(lib, shape, workspace, indices, F)
+        if need_dw:
+            _hot_measure(lib, shape, workspace, B, K, F, D, weight.dtype)
         if _check_indices:
             check_index_flag(dev)
     return loss, dvals, dbias, dW
@@ -908,7 +952,8 @@ def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, 
         if _hier_scratch_bytes != 0:
             B, K = indices.shape
             F, D = weight.shape
-            hot = bool(weight.requires_grad) and _use_hot_latents(B, K, F, D, weight.dtype)
+            hot = bool(weight.requires_grad) and _use_hot_latents(B, K, F, D, weight.dtype, weight.device,
+                                                                   _is_traced(weight))
             return hier_train_sliced(indices, weight, vals, bias, target, bool(weight.requires_grad), hot)[0]
     return hier_fwd(indices, weight, vals, bias, target)[0]
 

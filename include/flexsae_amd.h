@@ -245,6 +245,15 @@ size_t flexsae_hier_fwd_bwd_workspace_bytes_flags(const flexsae_shape *shape, in
  * (row, tile) walks that were deferred to the second pass, summed over the slices.
  */
 int flexsae_hier_hot_stats(const flexsae_shape *shape, const void *workspace, uint32_t *stats, void *stream);
+/*
+ * How skewed the indices of the last call on `workspace` were (any hierarchical backward / training
+ * step workspace whose pair list is complete; no counterpart in the reference): stats[0] = latents
+ * with more than 64 pairs, stats[1] = their 64-pair chunks, i.e. between 64 stats[1] - 63 stats[0] and
+ * 64 stats[1] of the B*K pairs belong to such latents.  `stats` may be device memory or pinned host
+ * memory (the kernel then writes across the bus and the caller polls an event: no synchronisation);
+ * a caller can use it to decide whether the next step is worth FLEXSAE_BWD_HOT_LATENTS.
+ */
+int flexsae_hier_pair_stats(const flexsae_shape *shape, const void *workspace, uint32_t *stats, void *stream);
 int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, const void *weight,
                          const void *vals, const void *bias, const void *target, float *loss,
                          void *dW, int dW_dtype, float *dvals, float *dbias, void *workspace,

@@ -135,3 +135,40 @@ def test_sgd_update_with_hot_latents():
     assert rel_err(Wn.double().cpu()[touched], want[touched]) <= 4e-3
     assert torch.equal(Wn.cpu()[~touched], cpu_args[1][~touched])
     assert abs(loss.item() - L) <= 1e-3 * abs(L) and rel_err(dv.cpu(), rv) <= 1e-2
+
+
+def test_auto_mode_follows_the_previous_step():
+    """"auto": the first step of a shape runs the plain kernel and leaves the skew of its indices in
+    pinned memory; the next step takes the accumulators for skewed indices and stays plain for
+    uniform ones.  Gradients match the oracle either way."""
+    import flexsae_amd as flex
+
+    print("[case] hot auto", flush=True)
+    flex.set_hot_latents("auto")
+    try:
+        for zipf, want_hot in ((1.1, True), (None, False)):
+            shape = (300, 64, 2000, 512) if zipf else (300, 64, 60000, 512)
+            cpu_args = make_inputs(*shape, torch.bfloat16, seed=34, zipf_s=zipf, unique=zipf is None, sort_vals=True,
+                                   w_std=0.3)
+            idx, W, v, b, t = _dev(cpu_args)
+            key = flex.ops._hot_key(W.device, *shape, torch.bfloat16)
+            grads = []
+            for step in range(3):
+                Wl = W.clone().requires_grad_()
+                loss = flex.triton_hierarchical_sae_loss(idx, Wl, v, b, t)
+                loss.backward()
+                torch.cuda.synchronize()
+                grads.append(Wl.grad)
+                # after a synchronisation the measurement is there for the next call to pick up
+                assert flex.ops._use_hot_latents(*shape, torch.bfloat16, W.device) == want_hot, (zipf, step)
+            assert flex.ops._hot_auto[key]["hot"] == want_hot
+            L, rW, _, _ = oracle.loss_grads(oracle.HIER, *cpu_args)
+            assert abs(loss.item() - L) <= 1e-3 * abs(L)
+            for g in grads:
+                assert rel_err(g.double().cpu(), rW) <= 1e-2
+            if want_hot:  # the first step ran the plain kernel, the later ones the accumulators
+                assert not torch.equal(grads[0], grads[1]) and torch.equal(grads[1], grads[2])
+            else:
+                assert torch.equal(grads[0], grads[1]) and torch.equal(grads[1], grads[2])
+    finally:
+        flex.set_hot_latents(None)
