@@ -926,7 +926,7 @@ void build_hot_tables(const flexsae_shape *s, const HierBwdPlan &pl, uint8_t *ws
                      reinterpret_cast<const uint32_t *>(ws + pl.off_slot), n_pairs);
   hipLaunchKernelGGL(hot_select_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count, sc.long_list, ctrl,
                      cand_list, long_cand, static_cast<uint32_t>(kHotMax));
-  hipLaunchKernelGGL(hot_mark_kernel, dim3(kHotMax), dim3(256), 0, st, begin, map, ctrl, cand_list, cand_state,
+  hipLaunchKernelGGL(hot_mark_kernel, dim3(kHotMax), dim3(1024), 0, st, begin, map, ctrl, cand_list, cand_state,
                      hot_list, hslot, static_cast<uint32_t>(s->K));
   hipLaunchKernelGGL(hot_cold_long_kernel, dim3(64), dim3(256), 0, st, sc.long_count, sc.long_list, long_cand,
                      cand_state, ctrl, long2);

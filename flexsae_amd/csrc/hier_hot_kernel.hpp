@@ -80,6 +80,7 @@ __global__ __launch_bounds__(1024) void hot_select_kernel(const uint32_t *__rest
   __shared__ uint32_t hist[256];
   __shared__ uint32_t cnt_lds[kCached];
   __shared__ uint32_t sel_prefix, sel_k, sel_prefix_next, sel_k_next, n_cand_s;
+  __shared__ uint32_t wave_tot[4];
   const int tid = threadIdx.x;
   const uint32_t n_long = *long_count;
   for (uint32_t i = tid; i < n_long && i < kCached; i += 1024) {
@@ -108,16 +109,28 @@ __global__ __launch_bounds__(1024) void hot_select_kernel(const uint32_t *__rest
         if (pass == 3 || (c >> hi_shift) == (prefix >> hi_shift)) atomicAdd(&hist[(c >> (8 * pass)) & 255u], 1u);
       }
       __syncthreads();
-      if (tid < 256) {
-        // the digit d with (entries above d) < k <= (entries above d) + hist[d]: every thread sums the
-        // bins above its own (broadcast reads) and exactly one finds itself selected (k is at most the
-        // number of entries counted in this pass)
-        uint32_t above = 0;
-        for (int d = tid + 1; d < 256; ++d) above += hist[d];
-        const uint32_t k = sel_k;
-        if (above < k && k <= above + hist[tid]) {
-          sel_k_next = k - above;
-          sel_prefix_next = prefix | (static_cast<uint32_t>(tid) << (8 * pass));
+      {
+        // the digit d with (entries above d) < k <= (entries above d) + hist[d]: a suffix sum over the
+        // 256 bins (shuffles inside each of the four wavefronts that hold them, then their totals);
+        // exactly one thread finds itself selected (k is at most the number of entries counted)
+        const int lane = tid & (kWave - 1), wv = tid >> 6;
+        const uint32_t h = tid < 256 ? hist[tid] : 0u;
+        uint32_t sfx = h;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+          const uint32_t y = __shfl_down(sfx, off, kWave);
+          if (lane + off < kWave) sfx += y;
+        }
+        if (lane == 0 && wv < 4) wave_tot[wv] = sfx;
+        __syncthreads();
+        if (tid < 256) {
+          uint32_t above = sfx - h;
+          for (int w = wv + 1; w < 4; ++w) above += wave_tot[w];
+          const uint32_t k = sel_k;
+          if (above < k && k <= above + h) {
+            sel_k_next = k - above;
+            sel_prefix_next = prefix | (static_cast<uint32_t>(tid) << (8 * pass));
+          }
         }
       }
       __syncthreads();
@@ -154,7 +167,7 @@ __global__ __launch_bounds__(1024) void hot_select_kernel(const uint32_t *__rest
 // accumulator then takes at most one addition per row, which the bound on its sums counts on); it
 // gets an accumulator row h and its pairs are marked in hslot[].  cand_state[c] = h or kHotNone.
 // hslot must hold a copy of slot[] on entry.
-__global__ __launch_bounds__(256) void hot_mark_kernel(const uint32_t *__restrict__ begin,
+__global__ __launch_bounds__(1024) void hot_mark_kernel(const uint32_t *__restrict__ begin,
                                                        const uint32_t *__restrict__ map,
                                                        uint32_t *__restrict__ ctrl,
                                                        const uint32_t *__restrict__ cand_list,
@@ -167,7 +180,7 @@ __global__ __launch_bounds__(256) void hot_mark_kernel(const uint32_t *__restric
   const uint32_t f = cand_list[c];
   const uint32_t s0 = begin[f], s1 = begin[f + 1];
   int dup = 0;
-  for (uint32_t i = s0 + threadIdx.x; i + 1 < s1; i += 256)  // the pair ids of a latent ascend
+  for (uint32_t i = s0 + threadIdx.x; i + 1 < s1; i += blockDim.x)  // the pair ids of a latent ascend
     dup |= (map[i] / K == map[i + 1] / K) ? 1 : 0;
   dup = __syncthreads_or(dup);
   if (threadIdx.x == 0) {
@@ -179,7 +192,7 @@ __global__ __launch_bounds__(256) void hot_mark_kernel(const uint32_t *__restric
   __syncthreads();
   const uint32_t h = h_s;
   if (h == kHotNone) return;
-  for (uint32_t i = s0 + threadIdx.x; i < s1; i += 256) hslot[map[i]] = kHotSlotBit | h;
+  for (uint32_t i = s0 + threadIdx.x; i < s1; i += blockDim.x) hslot[map[i]] = kHotSlotBit | h;
 }
 
 // long2_list = the latents with more than kSegChunk pairs that did not become hot (any order):

@@ -52,6 +52,9 @@ def _check_vs_oracle(cpu_args, dW, dv, db, loss, tol):
     ((260, 40, 1200, 384), torch.bfloat16, 1.1),     # K below the kernel's bound (per-step tests)
     ((384, 64, 1800, 256), torch.float16, 1.1),      # fp16 weights: fp32 contributions, fp32 dW
     ((2048, 64, 1000, 128), torch.bfloat16, 0.3),    # more long latents than accumulator rows
+    ((300, 64, 40000, 1536), torch.bfloat16, 1.1),   # most latents without a pair (the sparse reduction and its zero pass)
+    ((256, 32, 30000, 264), torch.bfloat16, 1.2),    # the same with a ragged last tile
+    ((384, 64, 50000, 256), torch.float16, 1.1),     # ... and an fp32 gradient of fp16 weights
 ])
 def test_hot_latents_match_the_oracle(shape, dtype, zipf):
     print("[case] hot", shape, dtype, zipf, flush=True)
