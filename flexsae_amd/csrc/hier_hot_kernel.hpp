@@ -27,21 +27,11 @@
 #include "hier_train_kernel.hpp"
 #include "segment_kernels.hpp"
 
-#ifndef FLEXSAE_HOT_EXP
-#define FLEXSAE_HOT_EXP 0
-#endif
-
 namespace flexsae {
 
 constexpr int kHotMax = 288;            // accumulator rows in the LDS: 288 * 128 columns * 4 bytes = 144 KiB
 constexpr int kHotCols = 128;           // columns per tile (two per lane)
-#ifndef FLEXSAE_HOT_DOT2
-#define FLEXSAE_HOT_DOT2 0
-#endif
-#ifndef FLEXSAE_HOT_THREADS
-#define FLEXSAE_HOT_THREADS 1024
-#endif
-constexpr int kHotThreads = FLEXSAE_HOT_THREADS;  // one block per compute unit: its LDS holds the accumulators
+constexpr int kHotThreads = 1024;       // one block per compute unit: its LDS holds the accumulators
 constexpr int kHotWaves = kHotThreads / kWave;
 constexpr int kHotRowsPerBlock = 128;   // fixed: the grouping of the sums must not depend on the slice width
 constexpr int kHotRowsPerWave = kHotRowsPerBlock / kHotWaves;
@@ -317,9 +307,6 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
   using raw_t = typename Piece::raw_t;
   using S_t = typename Traits<WT>::store_t;
   static_assert(sizeof(raw_t) == 4 && KMAX <= kWave && KMAX % 8 == 0, "16-bit weights, at most 64 steps");
-  // bf16 rows: the dvals dot product <w_k, S> runs on packed pairs (S rounded to bf16 for it, as the
-  // TopK backward does with its residual): one instruction per step instead of two
-  constexpr bool kDot2 = FLEXSAE_HOT_DOT2 && Traits<WT>::dtype == FLEXSAE_BF16;
   __shared__ int acc_lds[kHotMax * kHotCols];
   __shared__ int exp_lds[kHotWaves];
   __shared__ int ask_lds;   // the largest exponent a deferred row asked for
@@ -404,7 +391,7 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
 #pragma unroll
           for (int k = 0; k < KMAX; ++k) {
             if (FULL || k < kb) {  // uniform
-              const uint32_t row = FLEXSAE_HOT_EXP == 3 ? static_cast<uint32_t>(k) : static_cast<uint32_t>(bcast_i32(my_row, k));
+              const uint32_t row = static_cast<uint32_t>(bcast_i32(my_row, k));
               const auto dw = descriptor_load<sizeof(raw_t)>(row_descriptor(weight, row, w_row_bytes), w_lane_bytes);
               __builtin_memcpy(&raw[k], &dw, sizeof(raw_t));
             }
@@ -487,12 +474,11 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
               for (int c = 0; c < VEC; ++c) {
                 S[c] = fmaf(coef, e[c], S[c]);
                 contrib[c] = S[c] * v;
-                if (!kDot2) dot = fmaf(w[c], S[c], dot);
+                dot = fmaf(w[c], S[c], dot);
                 e[c] = fmaf(-w[c], v, e[c]);
               }
-              if constexpr (kDot2) dot = dot2_bf16(raw[k], f32x2_to_bf16x2_bits(S[0], S[1]), 0.f);
               const bool is_hot = (prow & kHotSlotBit) != 0;  // uniform: a pair of a hot latent
-              if (is_hot && hot_ok && FLEXSAE_HOT_EXP != 2) {
+              if (is_hot && hot_ok) {
                 int *a = my_acc + (prow & ~kHotSlotBit) * kHotCols;
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) {
@@ -510,11 +496,7 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
 #pragma unroll
                   for (int c = 0; c < VEC; ++c) packed[c] = __float_as_uint(contrib[c]);
                 }
-#if FLEXSAE_HOT_EXP != 1
                 descriptor_store<sizeof(packed), false>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
-#else
-                asm volatile("" ::"v"(packed[0]));
-#endif
               }
               dots[u] = dot;  // zero where the lane is beyond column D: its w is zero
             }

@@ -99,14 +99,8 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
   }
   const int64_t item = static_cast<int64_t>(blockIdx.x - fin.n_blocks) * (blockDim.x >> 6) + wave_in_block();
   if (item >= n_items) return;  // uniform per wavefront
-#ifdef FLEXSAE_TRAIN_ROW_MAJOR
-  const int n_t = static_cast<int>(n_items / B);
-  const int64_t b = item / n_t;
-  const int t = static_cast<int>(item - b * n_t);
-#else
   const int t = static_cast<int>(item / B);
   const int64_t b = item - static_cast<int64_t>(t) * B;
-#endif
   const int pc = t * (kWave * VEC) + lane * VEC;  // column inside the slice
   const int d0 = col0 + pc;
   const bool active = d0 < D;
