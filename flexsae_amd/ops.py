@@ -746,7 +746,11 @@ def hier_sgd_step(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, t
     with torch.cuda.device(dev):
         shape = _shape(B, K, F, D, weight, vals, bias.dtype, target.dtype)
         slice_cols = _hier_slice_cols(B, K, F, D, weight.dtype)
-        ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes(ctypes.byref(shape), slice_cols)
+        # hot-latent accumulators: the same decision as the loss takes (set_hot_latents)
+        hot_flag = _lib.BWD_HOT_LATENTS if _use_hot_latents(B, K, F, D, weight.dtype, dev, _is_traced(weight)) else 0
+        if hot_flag:
+            slice_cols = _hot_slice_cols(B, slice_cols, dev)
+        ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(shape), slice_cols, hot_flag)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         dvals = torch.empty((B, K), dtype=torch.float32, device=dev)
@@ -759,10 +763,13 @@ def hier_sgd_step(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, t
         rc = lib.flexsae_hier_sgd_step(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
                                        _ptr(target), _ptr(g), _ptr(loss), _ptr(dvals), _ptr(dbias),
                                        _ptr(workspace), ws_bytes,
-                                       _lib.BWD_REUSE_PAIR_LIST if cached is not None else 0, _ptr(flag), _stream())
+                                       (_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0) | hot_flag, _ptr(flag),
+                                       _stream())
         _lib.check(rc, "flexsae_hier_sgd_step")
         if cached is None:
             _pair_export(lib, shape, workspace, indices, F)
+        if not _is_traced(weight):
+            _hot_measure(lib, shape, workspace, B, K, F, D, weight.dtype)
         if _check_indices:
             check_index_flag(dev)
     return loss, dvals, dbias
