@@ -298,6 +298,39 @@ __device__ __forceinline__ void descriptor_store(__amdgpu_buffer_rsrc_t r, uint3
   else __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_bytes, 0, kAux);
 }
 
+// The same through a descriptor of a whole matrix of fewer than 4 GiB, the (wave-uniform) byte
+// offset of the row in a scalar register that the instruction adds by itself: where the row
+// offsets of all steps are computed at once by the lanes (one multiplication per lane) and read
+// back lane by lane, a gather or a store costs no address arithmetic at all.  No lane may lie
+// beyond its row: nothing is clipped at the row's end here.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t matrix_descriptor(const void *base, uint64_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0,
+                                           static_cast<int>(static_cast<uint32_t>(bytes)), 0x00020000);
+}
+template <int N>
+__device__ __forceinline__ vec_t<uint32_t, N / 4> descriptor_load_at(__amdgpu_buffer_rsrc_t r, uint32_t lane_bytes,
+                                                                     uint32_t row_bytes_offset) {
+  static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 bytes per lane");
+  if constexpr (N == 4) {
+    vec_t<uint32_t, 1> v;
+    v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, lane_bytes, row_bytes_offset, 0);
+    return v;
+  } else if constexpr (N == 8) {
+    return __builtin_amdgcn_raw_buffer_load_b64(r, lane_bytes, row_bytes_offset, 0);
+  } else {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, lane_bytes, row_bytes_offset, 0);
+  }
+}
+template <int N, bool NT = false>
+__device__ __forceinline__ void descriptor_store_at(__amdgpu_buffer_rsrc_t r, uint32_t lane_bytes,
+                                                    uint32_t row_bytes_offset, const vec_t<uint32_t, N / 4> &v) {
+  static_assert(N == 4 || N == 8 || N == 16, "4, 8 or 16 bytes per lane");
+  constexpr int kAux = NT ? 2 : 0;
+  if constexpr (N == 4) __builtin_amdgcn_raw_buffer_store_b32(v[0], r, lane_bytes, row_bytes_offset, kAux);
+  else if constexpr (N == 8) __builtin_amdgcn_raw_buffer_store_b64(v, r, lane_bytes, row_bytes_offset, kAux);
+  else __builtin_amdgcn_raw_buffer_store_b128(v, r, lane_bytes, row_bytes_offset, kAux);
+}
+
 // VEC consecutive elements of row `row` (wave-uniform) of a row-major matrix, starting at column
 // d0, as stored.  Lanes with d0 beyond the row get zeros.  Pieces of at least four bytes go
 // through a row descriptor (address arithmetic on the scalar unit).

@@ -592,9 +592,16 @@ void launch_train_hot_kernel(const flexsae_shape *s, const TrainArgs &ta, const 
     const int n_tiles = static_cast<int>(cols / kHotCols);
     const unsigned grid = static_cast<unsigned>(n_tiles) * static_cast<unsigned>(n_row_blocks);
     if (fin.mode != 0) fin.n_blocks = grid;  // every block takes a share
+    // 32-bit byte offsets from one descriptor per matrix where the matrices allow it
+    const bool off32 = s->D % kHotCols == 0 &&
+                       static_cast<uint64_t>(s->F) * s->D * sizeof(typename Traits<WT>::store_t) < (uint64_t{1} << 32) &&
+                       static_cast<uint64_t>(s->B) * s->K * slice_w * sizeof(typename Traits<PT>::store_t) < (uint64_t{1} << 31);
 #define FLEXSAE_TRAIN_HOT(KM)                                                                                   \
   do {                                                                                                          \
-    const auto kernel = s->K == KM ? hier_train_hot_kernel<WT, PT, KM, true> : hier_train_hot_kernel<WT, PT, KM, false>; \
+    const auto kernel = s->K == KM ? (off32 ? hier_train_hot_kernel<WT, PT, KM, true, true>                     \
+                                            : hier_train_hot_kernel<WT, PT, KM, true, false>)                   \
+                                   : (off32 ? hier_train_hot_kernel<WT, PT, KM, false, true>                    \
+                                            : hier_train_hot_kernel<WT, PT, KM, false, false>);                 \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kHotThreads), 0, st, indices, weight, vals, s->vals_dtype, ta.bias, \
                        s->bias_dtype, ta.target, s->target_dtype, coef, hslot, P, dvals, s_final, d_pad,        \
                        loss_partial, status_flag, s->B, n_tiles, n_row_blocks, col0, slice_w,                   \

@@ -292,7 +292,13 @@ __global__ __launch_bounds__(256) void hot_block_finalize_kernel(HotBlockFinaliz
 // of storing it.  The leading work of every block is its share of the previous slice's second
 // steps (fin, hfin); the last is the flush of its accumulators to
 // hot_partial[tile][row block][accumulator row][2][64].
-template <typename WT, typename PT, int KMAX, bool FULL>
+// OFF32: the weight matrix is smaller than 4 GiB, the slice of contributions smaller than 2 GiB
+// and D a whole number of tiles.  Rows and contribution rows are then addressed through one
+// descriptor each plus a 32-bit byte offset that the lanes compute for all steps of a row at once
+// (lane k: step k), so a step's gather and store need one lane read each and no scalar address
+// arithmetic; for a hot pair the same word carries the hot bit and the byte offset of its
+// accumulator row.  This kernel is bound by the instructions it issues, not by its bytes.
+template <typename WT, typename PT, int KMAX, bool FULL, bool OFF32>
 __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
     const int64_t *__restrict__ indices, const void *__restrict__ weight,
     const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
@@ -341,6 +347,8 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
   const uint32_t w_lane_bytes = static_cast<uint32_t>(d0) * sizeof(S_t);  // beyond the row if !active
   const uint32_t p_row_bytes = static_cast<uint32_t>(slice_w) * sizeof(typename Traits<PT>::store_t);
   const uint32_t p_lane_bytes = static_cast<uint32_t>(pc) * sizeof(typename Traits<PT>::store_t);
+  const __amdgpu_buffer_rsrc_t w_all = matrix_descriptor(weight, static_cast<uint64_t>(F) * w_row_bytes);
+  const __amdgpu_buffer_rsrc_t p_all = matrix_descriptor(P, static_cast<uint64_t>(B) * K * p_row_bytes);
   int *const my_acc = acc_lds + lane;  // element (i, lane) of accumulator row h is my_acc[h * 128 + i * 64]
 
   int exp_block = kHotExpMin;   // the block's exponent E (uniform over the block once set)
@@ -378,6 +386,14 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
           my_val = 0.f;
         }
         my_row = static_cast<int>(idx);
+        if constexpr (OFF32) {
+          // byte offsets instead of row numbers: of the weight row, and of the contribution row or
+          // (hot bit kept) of the accumulator row
+          my_row = static_cast<int>(static_cast<uint32_t>(my_row) * w_row_bytes);
+          const uint32_t sl = static_cast<uint32_t>(my_slot);
+          my_slot = static_cast<int>((sl & kHotSlotBit) ? (kHotSlotBit | ((sl & ~kHotSlotBit) * (kHotCols * 4u)))
+                                                        : sl * p_row_bytes);
+        }
         float tt[VEC];
         load_vec_dyn<WT, VEC>(bias, bias_dtype, dsafe, e);
         load_vec_dyn<WT, VEC>(target, target_dtype, b * D + dsafe, tt);
@@ -392,7 +408,8 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
           for (int k = 0; k < KMAX; ++k) {
             if (FULL || k < kb) {  // uniform
               const uint32_t row = static_cast<uint32_t>(bcast_i32(my_row, k));
-              const auto dw = descriptor_load<sizeof(raw_t)>(row_descriptor(weight, row, w_row_bytes), w_lane_bytes);
+              const auto dw = OFF32 ? descriptor_load_at<sizeof(raw_t)>(w_all, w_lane_bytes, row)
+                                    : descriptor_load<sizeof(raw_t)>(row_descriptor(weight, row, w_row_bytes), w_lane_bytes);
               __builtin_memcpy(&raw[k], &dw, sizeof(raw_t));
             }
           }
@@ -479,7 +496,8 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
               }
               const bool is_hot = (prow & kHotSlotBit) != 0;  // uniform: a pair of a hot latent
               if (is_hot && hot_ok) {
-                int *a = my_acc + (prow & ~kHotSlotBit) * kHotCols;
+                int *a = OFF32 ? reinterpret_cast<int *>(reinterpret_cast<char *>(my_acc) + (prow & ~kHotSlotBit))
+                               : my_acc + (prow & ~kHotSlotBit) * kHotCols;
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) {
                   // round(contrib * 2^(22 - E)) as an integer: |.| <= 2^22, so adding 1.5 * 2^23 leaves it in
@@ -496,7 +514,8 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
 #pragma unroll
                   for (int c = 0; c < VEC; ++c) packed[c] = __float_as_uint(contrib[c]);
                 }
-                descriptor_store<sizeof(packed), false>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
+                if constexpr (OFF32) descriptor_store_at<sizeof(packed), false>(p_all, p_lane_bytes, prow, packed);
+                else descriptor_store<sizeof(packed), false>(row_descriptor(P, prow, p_row_bytes), p_lane_bytes, packed);
               }
               dots[u] = dot;  // zero where the lane is beyond column D: its w is zero
             }
