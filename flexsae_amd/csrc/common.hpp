@@ -131,6 +131,46 @@ __device__ __forceinline__ float load_scalar(const void *base, int dtype, int64_
   return dtype == FLEXSAE_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
 }
 
+// The same in two halves, for code that wants several such loads in flight before it waits for
+// any of them: the bits as loaded (16-bit types in the low half), and their conversion.
+__device__ __forceinline__ uint32_t load_scalar_bits(const void *base, int dtype, int64_t i) {
+  if (dtype == FLEXSAE_F32) return static_cast<const uint32_t *>(base)[i];
+  return static_cast<const uint16_t *>(base)[i];
+}
+__device__ __forceinline__ float scalar_from_bits(uint32_t bits, int dtype) {
+  if (dtype == FLEXSAE_F32) return __uint_as_float(bits);
+  const uint16_t h = static_cast<uint16_t>(bits);
+  return dtype == FLEXSAE_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+}
+// two consecutive elements starting at an even element offset (the tensor's base 8-byte aligned)
+struct PairBits {
+  uint32_t lo, hi;
+};
+__device__ __forceinline__ PairBits load_pair_bits(const void *base, int dtype, int64_t off) {
+  PairBits r;
+  if (dtype == FLEXSAE_F32) {
+    const uint2 v = *reinterpret_cast<const uint2 *>(static_cast<const uint32_t *>(base) + off);
+    r.lo = v.x;
+    r.hi = v.y;
+  } else {
+    r.lo = *reinterpret_cast<const uint32_t *>(static_cast<const uint16_t *>(base) + off);
+    r.hi = 0u;
+  }
+  return r;
+}
+__device__ __forceinline__ void pair_from_bits(const PairBits &r, int dtype, float (&o)[2]) {
+  if (dtype == FLEXSAE_F32) {
+    o[0] = __uint_as_float(r.lo);
+    o[1] = __uint_as_float(r.hi);
+  } else if (dtype == FLEXSAE_BF16) {
+    o[0] = __uint_as_float(r.lo << 16);
+    o[1] = __uint_as_float(r.lo & 0xffff0000u);
+  } else {
+    o[0] = f16_bits_to_f32(static_cast<uint16_t>(r.lo));
+    o[1] = f16_bits_to_f32(static_cast<uint16_t>(r.lo >> 16));
+  }
+}
+
 // VEC consecutive elements of a run-time-typed tensor; takes the vector path when the
 // dtype equals the compile-time type T (the common case: all tensors share a dtype).
 template <typename T, int VEC>

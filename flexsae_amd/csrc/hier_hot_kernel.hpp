@@ -374,11 +374,20 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
       raw_t raw[KMAX];
       int exp_row = kHotExpMin;
       if (valid) {
-        int64_t idx = 0;
-        if (lane < K) {
-          idx = indices[pair0 + lane];
-          my_val = load_scalar(vals, vals_dtype, pair0 + lane);
-          my_slot = static_cast<int>(hslot[pair0 + lane]);
+        // everything the row needs before its gathers, requested at once and waited for once: a load
+        // issued after the stores of the row before it returns after them, so every separate wait here
+        // would cost a trip to memory of its own
+        const int64_t mine = pair0 + (lane < K ? lane : 0);
+        int64_t idx = indices[mine];
+        const uint32_t val_bits = load_scalar_bits(vals, vals_dtype, mine);
+        my_slot = static_cast<int>(hslot[mine]);
+        const PairBits bias_bits = load_pair_bits(bias, bias_dtype, dsafe);
+        const PairBits target_bits = load_pair_bits(target, target_dtype, b * D + dsafe);
+        my_val = scalar_from_bits(val_bits, vals_dtype);
+        if (lane >= K) {
+          idx = 0;
+          my_val = 0.f;
+          my_slot = 0;
         }
         if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(F)) {
           if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
@@ -395,8 +404,8 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
                                                         : sl * p_row_bytes);
         }
         float tt[VEC];
-        load_vec_dyn<WT, VEC>(bias, bias_dtype, dsafe, e);
-        load_vec_dyn<WT, VEC>(target, target_dtype, b * D + dsafe, tt);
+        pair_from_bits(bias_bits, bias_dtype, e);
+        pair_from_bits(target_bits, target_dtype, tt);
 #pragma unroll
         for (int c = 0; c < VEC; ++c) {
           e[c] -= tt[c];
