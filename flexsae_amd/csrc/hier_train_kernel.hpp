@@ -114,19 +114,46 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     return kb;
   };
 
+  // Everything the row needs before its gathers is requested at once and waited for once: the
+  // conversions branch on run-time dtypes, and a wait inside each of them made this a chain of
+  // five or six trips to memory, one after the other, before the first gather was issued.
   int my_row[KC], my_slot[KC];
   float my_val[KC], my_dval[KC];
+  int64_t idx_bits[KC];
+  uint32_t val_bits[KC];
 #pragma unroll
   for (int c = 0; c < KC; ++c) {
     const int kk = c * kWave + lane;
-    int64_t idx = 0;
-    my_val[c] = 0.f;
-    my_slot[c] = 0;
+    const int64_t mine = pair0 + (kk < K ? kk : 0);
+    idx_bits[c] = indices[mine];
+    val_bits[c] = load_scalar_bits(vals, vals_dtype, mine);
+    my_slot[c] = static_cast<int>(slot[mine]);
+  }
+  // bias - target before the gathers: the memory counter retires in order, so a load issued after
+  // the gathers could only be waited for together with all of them
+  float e[VEC], tt[VEC], acc[VEC];
+  if constexpr (VEC == 2) {
+    const PairBits bias_bits = load_pair_bits(bias, bias_dtype, dsafe);
+    const PairBits target_bits = load_pair_bits(target, target_dtype, b * D + dsafe);
+    pair_from_bits(bias_bits, bias_dtype, e);
+    pair_from_bits(target_bits, target_dtype, tt);
+  } else {
+    static_assert(VEC == 1, "one or two columns per lane");
+    const uint32_t bias_bits = load_scalar_bits(bias, bias_dtype, dsafe);
+    const uint32_t target_bits = load_scalar_bits(target, target_dtype, b * D + dsafe);
+    e[0] = scalar_from_bits(bias_bits, bias_dtype);
+    tt[0] = scalar_from_bits(target_bits, target_dtype);
+  }
+#pragma unroll
+  for (int c = 0; c < KC; ++c) {
+    const int kk = c * kWave + lane;
+    int64_t idx = idx_bits[c];
+    my_val[c] = scalar_from_bits(val_bits[c], vals_dtype);
     my_dval[c] = 0.f;
-    if (kk < K) {
-      idx = indices[pair0 + kk];
-      my_val[c] = load_scalar(vals, vals_dtype, pair0 + kk);
-      my_slot[c] = static_cast<int>(slot[pair0 + kk]);
+    if (kk >= K) {
+      idx = 0;
+      my_val[c] = 0.f;
+      my_slot[c] = 0;
     }
     if (static_cast<uint64_t>(idx) >= static_cast<uint64_t>(F)) {
       if (status_flag) atomicOr(status_flag, FLEXSAE_FLAG_INDEX_RANGE);
@@ -135,12 +162,6 @@ __global__ __launch_bounds__(256) void hier_train_kernel(
     }
     my_row[c] = static_cast<int>(idx);
   }
-
-  // bias - target first: the memory counter retires in order, so a load issued after the gathers
-  // could only be waited for together with all of them
-  float e[VEC], tt[VEC], acc[VEC];
-  load_vec_dyn<WT, VEC>(bias, bias_dtype, dsafe, e);
-  load_vec_dyn<WT, VEC>(target, target_dtype, b * D + dsafe, tt);
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
     e[i] -= tt[i];
