@@ -720,6 +720,23 @@ def test_topk_residual_precision_switch():
     _check_against_oracle("topk", args, torch.bfloat16, 0.7, got, ref_tols=False)
 
 
+def test_topk_workspace_query_covers_both_residual_layouts():
+    """bf16 weights, K = 512: the fp32-residual variant works on narrower tiles and needs more room
+    for its per-tile shares of dvals than the bf16 one; the size query takes no flags and must
+    cover both, so the same workspace serves either call."""
+    B, K, F, D = 64, 512, 2048, 512
+    args = make_inputs(B, K, F, D, dtype=torch.bfloat16, seed=29)
+    L, rW, rv, rb = oracle.loss_grads(oracle.TOPK, *args, grad_out=1.0)
+    idx, W, v, b, t = _to_dev(args)
+    rc, loss, resid = abi.forward("topk", idx, W, v, b, t)
+    assert rc == 0
+    for flags, tol in ((0, 1e-2), (abi._lib.TOPK_BWD_FP32_RESIDUAL, 1e-4)):
+        rc, dW, dv, db = abi.topk_backward(idx, W, v, resid, 1.0, dw_dtype=torch.float32, flags=flags)
+        torch.cuda.synchronize()
+        assert rc == 0, abi._lib.status_string(rc)
+        assert rel_err(dW.cpu(), rW) < tol and rel_err(dv.cpu(), rv) < tol and rel_err(db.cpu(), rb) < 1e-4
+
+
 def test_topk_target_gradient():
     args = make_inputs(16, 8, 40, 256, seed=2)
     idx, W, v, b, t = _to_dev(args)
