@@ -59,10 +59,11 @@ def hier_backward(indices, weight, vals, resid, grad_out, flag=None, slice_cols=
 
 
 def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_dtype=torch.float32, flags=0,
-               alloc_dw=True, keep_workspace=False):
+               alloc_dw=True, keep_workspace=False, workspace=None):
     """Fused forward+backward for a unit upstream gradient -> (rc, loss, dW, dvals, dbias);
     ``alloc_dw=False`` passes a null dW (for FLEXSAE_BWD_NO_DW); ``keep_workspace`` appends the
-    workspace to the result (for flexsae_hier_hot_stats)."""
+    workspace to the result (for flexsae_hier_hot_stats); ``workspace`` is one kept from an earlier
+    call (for the reuse flags)."""
     lib = _lib.load()
     sh = shape_of(indices, weight, vals, bias.dtype, target.dtype)
     dev = weight.device
@@ -73,7 +74,8 @@ def hier_train(indices, weight, vals, bias, target, flag=None, slice_cols=0, dw_
     # slices of whole training tiles where the entry point supports the shape
     nbytes = (lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(sh), slice_cols, flags)
               or lib.flexsae_hier_bwd_workspace_bytes(ctypes.byref(sh), slice_cols))
-    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    ws = workspace if workspace is not None else torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    assert ws.numel() >= nbytes
     rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(sh), ptr(indices), ptr(weight), ptr(vals), ptr(bias), ptr(target),
                                   ptr(loss), ptr(dW), DT[dw_dtype], ptr(dv), ptr(db), ptr(ws), nbytes, flags,
                                   ptr(flag), stream())

@@ -123,6 +123,60 @@ def test_deferred_rows_and_reproducibility():
         _check_vs_oracle(cpu_args, outs[0], dv, db, loss, 1e-2)
 
 
+def test_pair_list_and_hot_tables_reused():
+    """A second call on the same workspace may keep the pair list (FLEXSAE_BWD_REUSE_PAIR_LIST: the hot
+    tables are rebuilt from it) and the hot tables too (FLEXSAE_BWD_REUSE_HOT_TABLES): the same bits
+    either way, also for other values and targets on the same indices."""
+    print("[case] hot reuse", flush=True)
+    cpu_args = make_inputs(300, 64, 2000, 512, torch.bfloat16, seed=34, zipf_s=1.1, sort_vals=True, w_std=0.3)
+    idx, W, v, b, t = _dev(cpu_args)
+    rc, loss0, dW0, dv0, db0, ws = abi.hier_train(idx, W, v, b, t, dw_dtype=torch.bfloat16, slice_cols=256, flags=HOT,
+                                                   keep_workspace=True)
+    assert rc == 0 and abi.hot_stats(idx, W, v, b, t, ws)[0] > 0
+    v2, t2 = (v.float() * 0.5 + 0.1).to(v.dtype), (t.float() * 1.5).to(t.dtype)
+    rc, loss1, dW1, dv1, db1 = abi.hier_train(idx, W, v2, b, t2, dw_dtype=torch.bfloat16, slice_cols=256, flags=HOT)
+    assert rc == 0
+    for reuse in (_lib.BWD_REUSE_PAIR_LIST, _lib.BWD_REUSE_PAIR_LIST | _lib.BWD_REUSE_HOT_TABLES):
+        for (vv, tt), want in (((v, t), (loss0, dW0, dv0, db0)), ((v2, t2), (loss1, dW1, dv1, db1))):
+            rc, loss, dW, dv, db = abi.hier_train(idx, W, vv, b, tt, dw_dtype=torch.bfloat16, slice_cols=256,
+                                                  flags=HOT | reuse, workspace=ws)
+            assert rc == 0, _lib.status_string(rc)
+            assert torch.equal(loss, want[0]) and torch.equal(dW, want[1])
+            assert torch.equal(dv, want[2]) and torch.equal(db, want[3])
+
+
+def test_hot_latents_under_a_shared_pair_list():
+    """Through the package: both losses inside shared_pair_list() with the hot path forced on give
+    the gradients of separate calls, bit for bit."""
+    import flexsae_amd as flex
+    print("[case] hot shared pair list", flush=True)
+    cpu_args = make_inputs(512, 64, 3000, 512, torch.bfloat16, seed=35, zipf_s=1.1, sort_vals=True, w_std=0.3)
+
+    def grads(shared):
+        idx, W, v, b, t = _dev(cpu_args)
+        W.requires_grad_(); v.requires_grad_(); b.requires_grad_()
+        import contextlib
+        with (flex.shared_pair_list() if shared else contextlib.nullcontext()):
+            (flex.triton_hierarchical_sae_loss(idx, W, v, b, t) + flex.triton_topk_sae_loss(idx, W, v, b, t)).backward()
+        return W.grad, v.grad, b.grad
+
+    flex.set_hot_latents("on")
+    try:
+        a, b_ = grads(False), grads(True)
+    finally:
+        flex.set_hot_latents("auto")
+    for x, y in zip(a, b_):
+        assert torch.equal(x, y)
+    # and the hot path was what ran: differs from the plain step in dW only by rounding
+    flex.set_hot_latents("off")
+    try:
+        c = grads(False)
+    finally:
+        flex.set_hot_latents("auto")
+    assert not torch.equal(a[0], c[0]) and rel_err(a[0].float().cpu(), c[0].float().cpu()) < 1e-2
+    assert torch.equal(a[1], c[1])
+
+
 def test_sgd_update_with_hot_latents():
     print("[case] hot sgd", flush=True)
     cpu_args = make_inputs(300, 64, 2000, 512, torch.bfloat16, seed=33, zipf_s=1.1, sort_vals=True, w_std=0.3)
