@@ -177,6 +177,58 @@ def test_hot_latents_under_a_shared_pair_list():
     assert torch.equal(a[1], c[1])
 
 
+def test_hot_step_in_a_graph():
+    """The step with the hot path forced on, recorded into a HIP graph and replayed with other
+    indices (another set of frequent latents) and values, eager work between the replays: every
+    replay equals the eager step on the same inputs, bit for bit.  Selection, marking and the
+    accumulators' exponents all live on the device, so nothing of them is frozen into the graph."""
+    import flexsae_amd as flex
+    print("[case] hot graph", flush=True)
+    shape = (300, 64, 2000, 512)
+    mk = lambda seed: make_inputs(*shape, torch.bfloat16, seed=seed, zipf_s=1.1, sort_vals=True, w_std=0.3)
+    idx, W, v, b, t = _dev(mk(40))
+    W.requires_grad_(); v.requires_grad_(); b.requires_grad_()
+
+    def step():
+        W.grad = v.grad = b.grad = None
+        loss = flex.triton_hierarchical_sae_loss(idx, W, v, b, t)
+        loss.backward()
+        return loss
+
+    flex.set_hot_latents("on")
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        W.grad = v.grad = b.grad = None
+        with torch.cuda.graph(graph):
+            static_loss = flex.triton_hierarchical_sae_loss(idx, W, v, b, t)
+            static_loss.backward()
+        for trial in range(3):
+            new = mk(41 + trial)
+            with torch.no_grad():
+                for dst, src in zip((idx, W, v, b, t), new):
+                    dst.copy_(src.to(DEV))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = (static_loss.clone(), W.grad.clone(), v.grad.clone(), b.grad.clone())
+            i2, W2, v2, b2, t2 = _dev(new)  # eager work between the replays
+            W2.requires_grad_(); v2.requires_grad_(); b2.requires_grad_()
+            loss2 = flex.triton_hierarchical_sae_loss(i2, W2, v2, b2, t2)
+            loss2.backward()
+            for a, c in zip(got, (loss2.detach(), W2.grad, v2.grad, b2.grad)):
+                assert torch.equal(a, c), trial
+            L, rW, rv, rb = oracle.loss_grads(oracle.HIER, *new)
+            assert rel_err(got[1].double().cpu(), torch.from_numpy(rW)) <= 1e-2
+    finally:
+        flex.set_hot_latents("auto")
+
+
 def test_sgd_update_with_hot_latents():
     print("[case] hot sgd", flush=True)
     cpu_args = make_inputs(300, 64, 2000, 512, torch.bfloat16, seed=33, zipf_s=1.1, sort_vals=True, w_std=0.3)
