@@ -310,14 +310,17 @@ def main():
     slice_cols = D if staged else flex.ops._hier_slice_cols(B, K, F, D, dtype)
     # hot-latent accumulators: the same decision as the API takes for a weight that needs its gradient
     hot = bool(fused and not staged and flex.ops._use_hot_latents(B, K, F, D, dtype, dev))
-    HOTF = _lib.BWD_HOT_LATENTS if hot else 0
+    # ... and whether shapes with few pairs per latent reduce without the row-count list
+    dense = bool(fused and not staged and flex.ops._use_dense_latents(B, K, F, D, dtype, dev))
+    HOTF = (_lib.BWD_HOT_LATENTS if hot else 0) | (_lib.BWD_DENSE_LATENTS if dense else 0)
     if hot:
         slice_cols = flex.ops._hot_slice_cols(B, slice_cols, dev)
     tile = 64 * (4 if D % 4 == 0 else 2 if D % 2 == 0 else 1)
     d_pad = -(-D // tile) * tile
     if fused:
         # slices are whole training tiles when the reduction can work on 256-byte pieces
-        bws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(sh), slice_cols, HOTF)
+        bws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(sh), slice_cols,
+                                                                   _lib.BWD_HOT_LATENTS if hot else 0)
         train_tile = 64 if (dtype == torch.float32 and K > 64) else 128
         granule = train_tile if D % (16 // p_size) == 0 else tile
     else:
@@ -461,7 +464,7 @@ def main():
         "build_id": build_id,
         "config": {"workload": f"HierarchicalTopK fwd+bwd, {args.workload}: B={B} K={K} F={F} D={D} {dt_name}, "
                                f"indices {dist}", "B": B, "K": K, "F": F, "D": D,
-                   "hier_scratch_mb": scratch >> 20, "hier_slice_cols": int(slice_w), "hot_latents": hot, "fused_training_step": bool(fused), "hier_mode": hier_mode,
+                   "hier_scratch_mb": scratch >> 20, "hier_slice_cols": int(slice_w), "hot_latents": hot, "dense_latents": dense, "fused_training_step": bool(fused), "hier_mode": hier_mode,
                    "hier_stage_mb": flex.ops.hier_stage_bytes(dev) >> 20},
         "roofline": roofline,
         "step_hbm": {"algorithmic_bytes": abytes["hier_step"],

@@ -8,7 +8,8 @@ as hand-written HIP kernels for AMD MI355X (gfx950), behind the reference packag
 Public names mirror reference torch-ext/flex_sae/__init__.py:5-18.  The ``triton_*`` names are
 kept so that existing callers need no edit; nothing here uses Triton.
 """
-from .ops import (check_index_flag, hier_stage_bytes, hierarchical_sae_sgd_step, set_fused_training,
+from .ops import (check_index_flag, hier_stage_bytes, hierarchical_sae_sgd_step, set_dense_latents,
+                  set_fused_training,
                   set_hier_min_slice_cols, set_hier_scratch_bytes, set_hier_stage_bytes, set_hot_latents,
                   set_index_checking, set_topk_residual_bf16, shared_pair_list, triton_hierarchical_sae_loss,
                   triton_topk_sae_loss)
@@ -41,6 +42,7 @@ __all__ = [
     "hier_stage_bytes",
     "set_fused_training",
     "set_hot_latents",
+    "set_dense_latents",
     "set_topk_residual_bf16",
     "shared_pair_list",
 ]

@@ -36,6 +36,7 @@ BWD_SKIP_EPILOGUE = 64
 BWD_HOT_LATENTS = 128
 BWD_HOT_NO_HEADROOM = 512
 BWD_REUSE_HOT_TABLES = 1024
+BWD_DENSE_LATENTS = 2048
 TOPK_BWD_FP32_RESIDUAL = 256
 
 

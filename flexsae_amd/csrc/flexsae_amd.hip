@@ -382,7 +382,13 @@ static_assert(kSegClasses + 1 <= kClsStride, "a counter array holds one slot per
 
 // Most latents without a pair, the rest with few: the reduction by pieces then works from the list
 // of latents ordered by row count and the rows of latents without pairs are zeroed in one pass.
-inline bool sparse_latents(const flexsae_shape *s) { return s->B * s->K <= 2 * s->F; }
+// Whether that pays depends on how many latents really are without a pair: with two pairs per latent
+// on average it does for skewed indices (two thirds of the latents empty: the step a sixth faster) and
+// does not for uniform ones (an eighth of them empty: the step 8 % slower).  Only the caller can know,
+// from an earlier step: FLEXSAE_BWD_DENSE_LATENTS says "most latents have pairs".
+inline bool sparse_latents(const flexsae_shape *s, int flags = 0) {
+  return !(flags & FLEXSAE_BWD_DENSE_LATENTS) && s->B * s->K <= 2 * s->F;
+}
 
 struct HierBwdPlan {
   int vec;                 // columns per lane
@@ -764,7 +770,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   // Sparse shapes reduce every slice by pieces from the list of latents ordered by row count; the
   // rows of latents without pairs are zeroed here, whole rows in one pass (the in-place update leaves
   // them alone).
-  const bool sparse = piece != 0 && sparse_latents(s);
+  const bool sparse = piece != 0 && sparse_latents(s, flags);
   const uint32_t *cls_begin = reinterpret_cast<const uint32_t *>(ws + pl.off_cls) + 2 * kClsStride;
   const uint32_t *cls_list = reinterpret_cast<const uint32_t *>(ws + pl.off_cls_list);
   if (sparse && do_reduce && !update)
@@ -816,7 +822,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     // of the four latents a wavefront would otherwise share (4 % faster on slices read from HBM).
     const bool cache_sized = static_cast<size_t>(s->B * s->K) * static_cast<size_t>(sw) * pl.p_size <= (size_t{384} << 20);
     const bool by_pieces =
-        piece != 0 && (update || cols % pl.tile != 0 || s->B * s->K <= 2 * s->F || cache_sized);
+        piece != 0 && (update || cols % pl.tile != 0 || sparse_latents(s, flags) || cache_sized);
     launch_seg_reduce<PT, GT, VEC>(narrow_reduce, begin, sc_cold, chunk_begin, P, partial, dW, dw_scale, s->F, tps,
                                    static_cast<int>(col0), sw, D, st, by_pieces ? piece : 0, cols, s->B * s->K, update,
                                    sparse ? cls_begin : nullptr, sparse ? cls_list : nullptr, fold ? &pending : nullptr);
@@ -902,9 +908,9 @@ void launch_hier_slices_w(const flexsae_shape *s, const HierBwdPlan &pl, int64_t
 // What follows the pair list in a hierarchical workspace: the chunk table of the hot latents and, for
 // sparse shapes, the list of latents ordered by row count.
 void finish_pair_list(const flexsae_shape *s, const HierBwdPlan &pl, uint8_t *ws, const uint32_t *begin,
-                      const CsrScratch &sc, hipStream_t st) {
+                      const CsrScratch &sc, hipStream_t st, int flags = 0) {
   uint32_t *cls = reinterpret_cast<uint32_t *>(ws + pl.off_cls);
-  const bool sparse = sparse_latents(s);
+  const bool sparse = sparse_latents(s, flags);
   hipLaunchKernelGGL(seg_chunk_table_kernel, dim3(1), dim3(1024), 0, st, begin, sc.long_count, sc.long_list,
                      reinterpret_cast<uint32_t *>(ws + pl.off_chunk), sparse ? cls : static_cast<uint32_t *>(nullptr),
                      2 * kClsStride);
@@ -1203,7 +1209,8 @@ int flexsae_hier_pair_stats(const flexsae_shape *s, const void *workspace, uint3
   const HierBwdPlan pl = plan_hier_bwd(s);  // the part of the layout every hierarchical workspace shares
   uint8_t *ws = static_cast<uint8_t *>(const_cast<void *>(workspace));
   const CsrScratch sc = carve_csr_scratch(ws + pl.off_csr, s->F, s->B * s->K);
-  hipLaunchKernelGGL(pair_stats_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), sc.long_count,
+  hipLaunchKernelGGL(pair_stats_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<const uint32_t *>(ws + pl.off_begin), s->F, sc.long_count,
                      reinterpret_cast<const uint32_t *>(ws + pl.off_chunk), stats);
   return launch_status();
 }
@@ -1260,7 +1267,7 @@ int flexsae_hier_bwd(const flexsae_shape *s, const int64_t *indices, const void 
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
     csr_build_launch(indices, s->B, s->K, s->F, begin, map, reinterpret_cast<uint32_t *>(ws + pl.off_slot), sc,
                      status_flag, st);
-    finish_pair_list(s, pl, ws, begin, sc, st);
+    finish_pair_list(s, pl, ws, begin, sc, st, flags);
   }
   const float coef = static_cast<float>(
       2.0 / (static_cast<double>(s->B) * static_cast<double>(s->K) * static_cast<double>(s->D)));
@@ -1374,7 +1381,7 @@ int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void
   if (!(flags & FLEXSAE_BWD_REUSE_PAIR_LIST)) {
     csr_build_launch(indices, s->B, s->K, s->F, begin, map, reinterpret_cast<uint32_t *>(ws + pl.off_slot), sc,
                      status_flag, st);
-    finish_pair_list(s, pl, ws, begin, sc, st);
+    finish_pair_list(s, pl, ws, begin, sc, st, flags);
   }
   if (hot && !((flags & FLEXSAE_BWD_REUSE_PAIR_LIST) && (flags & FLEXSAE_BWD_REUSE_HOT_TABLES)))
     build_hot_tables(s, pl, ws, sc, st);
@@ -1386,7 +1393,7 @@ int hier_fwd_bwd_impl(const flexsae_shape *s, const int64_t *indices, const void
   launch_hier_slices_w<4>(s, pl, slice_w, indices, weight, vals, nullptr, sgd_step, coef, dW,
                           no_dw ? s->weight_dtype : dW_dtype, dvals, dbias, ws,
                           (flags & (FLEXSAE_BWD_SWEEP_ONLY | FLEXSAE_BWD_REDUCE_ONLY | FLEXSAE_BWD_SKIP_EPILOGUE |
-                                    FLEXSAE_BWD_HOT_NO_HEADROOM)) |
+                                    FLEXSAE_BWD_HOT_NO_HEADROOM | FLEXSAE_BWD_DENSE_LATENTS)) |
                               (no_dw ? FLEXSAE_BWD_SWEEP_ONLY : 0) | (sgd_step ? kBwdSgdUpdate : 0) | (hot ? kBwdHot : 0),
                           status_flag, st, &ta, piece ? static_cast<int>(piece_cols(pl)) : 0);
   return launch_status();
@@ -1412,7 +1419,7 @@ int flexsae_hier_sgd_step(const flexsae_shape *s, const int64_t *indices, void *
   return hier_fwd_bwd_impl(s, indices, weight, vals, bias, target, loss, weight, s->weight_dtype, dvals, dbias,
                            workspace, workspace_bytes,
                            flags & (FLEXSAE_BWD_REUSE_PAIR_LIST | FLEXSAE_BWD_HOT_LATENTS | FLEXSAE_BWD_REUSE_HOT_TABLES |
-                                    FLEXSAE_BWD_HOT_NO_HEADROOM),
+                                    FLEXSAE_BWD_HOT_NO_HEADROOM | FLEXSAE_BWD_DENSE_LATENTS),
                            status_flag, stream, step);
 }
 

@@ -201,14 +201,29 @@ __global__ void hot_cold_long_kernel(const uint32_t *__restrict__ long_count,
   }
 }
 
-// out[0] = latents with more than kSegChunk pairs, out[1] = their 64-pair chunks (so between
-// out[1] * 64 - 63 * out[0] and out[1] * 64 pairs belong to them).  `out` may be pinned host memory.
-__global__ void pair_stats_kernel(const uint32_t *__restrict__ long_count, const uint32_t *__restrict__ chunk_begin,
-                                  uint32_t *__restrict__ out) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
+// out[0] = latents with more than kSegChunk pairs, out[1] = their pairs in chunks of kSegChunk,
+// out[2] = latents without a pair.  One block (the pair list's segment starts are read once:
+// 4 bytes per latent); `out` may be pinned host memory.
+__global__ __launch_bounds__(1024) void pair_stats_kernel(const uint32_t *__restrict__ begin, int64_t F,
+                                                          const uint32_t *__restrict__ long_count,
+                                                          const uint32_t *__restrict__ chunk_begin,
+                                                          uint32_t *__restrict__ out) {
+  __shared__ uint32_t wave_tot[1024 / kWave];
+  uint32_t mine = 0;  // per lane, so that the loads of several rounds are in flight together
+#pragma unroll 8
+  for (int64_t f = threadIdx.x; f < F; f += 1024) mine += begin[f + 1] == begin[f] ? 1u : 0u;
+  uint32_t empty = mine;
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) empty += static_cast<uint32_t>(__shfl_xor(static_cast<int>(empty), off, kWave));
+  if (lane_id() == 0) wave_tot[threadIdx.x >> 6] = empty;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t total = 0;
+    for (int w = 0; w < 1024 / kWave; ++w) total += wave_tot[w];
     const uint32_t n_long = *long_count;
     out[0] = n_long;
     out[1] = chunk_begin[n_long];
+    out[2] = total;
   }
 }
 

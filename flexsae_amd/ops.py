@@ -245,10 +245,21 @@ def set_hier_scratch_bytes(nbytes) -> None:
 # shape on the same device takes the accumulators when that was a quarter of the pairs or more.  The
 # first step of a shape, and steps traced by a compiler, run the plain kernel.
 # "on" takes them wherever the shape is supported (16-bit weights, K <= 64); "off" never.
+#
+# The same measurement serves a second decision (FLEXSAE_BWD_DENSE_LATENTS of the library).  Shapes
+# with at most two pairs per latent on average (B*K <= 2F) reduce, by default, from a list of the
+# latents ordered by pair count and zero the rows of latents without pairs in one pass: a sixth faster
+# where two thirds of the latents are empty (skewed indices), 8 % slower where an eighth is (uniform
+# ones; B = 4096, K = 32, F = 65536: 0.441 instead of 0.477 ms without the list).  The step therefore
+# also leaves the number of latents without pairs, and the next one drops the list when that was less
+# than 40 % of the latents (with uniform indices the two ways break even at one pair per latent, 37 %
+# empty).
 _hot_latents = os.environ.get("FLEXSAE_HOT_LATENTS", "auto").lower()
+_dense_latents = os.environ.get("FLEXSAE_DENSE_LATENTS", "auto").lower()
 _HOT_ROWS_PER_BLOCK = 128   # kHotRowsPerBlock of the library
 _HOT_AUTO_FRACTION = 0.25   # of the pairs in latents with more than 64 pairs
-_hot_auto = {}              # (device index, B, K, F, D, dtype) -> {"hot", "pinned", "event"}
+_DENSE_AUTO_FRACTION = 0.40  # of the latents without a pair
+_hot_auto = {}              # (device index, B, K, F, D, dtype) -> {"hot", "dense", "pinned", "event"}
 
 
 def set_hot_latents(mode) -> None:
@@ -263,6 +274,21 @@ def set_hot_latents(mode) -> None:
     if mode not in ("auto", "on", "off"):
         raise ValueError("set_hot_latents: expected 'auto', 'on' or 'off'")
     _hot_latents = mode
+    _hot_auto.clear()
+
+
+def set_dense_latents(mode) -> None:
+    """``"auto"`` (default), ``"on"``/``True`` or ``"off"``/``False``: whether the sliced hierarchical
+    step of a shape with at most two pairs per latent (B*K <= 2F) reduces WITHOUT the list of latents
+    ordered by pair count (``"on"``: most latents have pairs).  The results are the same bits either
+    way.  ``"auto"`` decides from the previous step of the same shape (see the module's comment)."""
+    global _dense_latents
+    if isinstance(mode, bool):
+        mode = "on" if mode else "off"
+    mode = "auto" if mode is None else str(mode).lower()
+    if mode not in ("auto", "on", "off"):
+        raise ValueError("set_dense_latents: expected 'auto', 'on' or 'off'")
+    _dense_latents = mode
     _hot_auto.clear()
 
 
@@ -285,26 +311,45 @@ def _use_hot_latents(B: int, K: int, F: int, D: int, weight_dtype, device=None, 
         return True
     if traced or device is None or torch.cuda.is_current_stream_capturing():
         return False  # (a graph under capture keeps whatever kernel it captured)
-    st = _hot_auto.get(_hot_key(device, B, K, F, D, weight_dtype))
-    if st is None:
+    st = _index_stats(_hot_key(device, B, K, F, D, weight_dtype), B, K, F)
+    return st is not None and st["hot"]
+
+
+def _use_dense_latents(B: int, K: int, F: int, D: int, weight_dtype, device=None, traced: bool = False) -> bool:
+    if B * K > 2 * F or _dense_latents == "off":
+        return False  # (with more pairs than that the library never uses the list)
+    if _dense_latents == "on":
+        return True
+    if traced or device is None or torch.cuda.is_current_stream_capturing():
         return False
+    st = _index_stats(_hot_key(device, B, K, F, D, weight_dtype), B, K, F)
+    return st is not None and st["dense"]
+
+
+def _index_stats(key, B, K, F):
+    """What the last measured step of the shape said about its indices (None: nothing yet)."""
+    st = _hot_auto.get(key)
+    if st is None:
+        return None
     if st["event"] is not None and st["event"].query():  # the previous step's measurement has arrived
         long_pairs = int(st["pinned"][1]) * 64
         st["hot"] = long_pairs >= _HOT_AUTO_FRACTION * B * K
+        st["dense"] = int(st["pinned"][2]) < _DENSE_AUTO_FRACTION * F
         st["event"] = None
-    return st["hot"]
+    return st
 
 
 def _hot_measure(lib, shape, workspace: Tensor, B, K, F, D, weight_dtype) -> None:
     """Leave the skew of this step's indices where the next step of the shape finds it."""
-    if _hot_latents != "auto" or not _hot_latents_supported(B, K, F, D, weight_dtype):
-        return
-    if torch.cuda.is_current_stream_capturing():
+    wanted = ((_hot_latents == "auto" and _hot_latents_supported(B, K, F, D, weight_dtype))
+              or (_dense_latents == "auto" and B * K <= 2 * F))
+    if not wanted or torch.cuda.is_current_stream_capturing():
         return
     key = _hot_key(workspace.device, B, K, F, D, weight_dtype)
     st = _hot_auto.get(key)
     if st is None:
-        st = _hot_auto[key] = {"hot": False, "pinned": torch.zeros(2, dtype=torch.int32, pin_memory=True), "event": None}
+        st = _hot_auto[key] = {"hot": False, "dense": False,
+                               "pinned": torch.zeros(3, dtype=torch.int32, pin_memory=True), "event": None}
     if st["event"] is not None:
         return  # a measurement is still on its way
     rc = lib.flexsae_hier_pair_stats(ctypes.byref(shape), _ptr(workspace), _ptr(st["pinned"]), _stream())
@@ -660,14 +705,16 @@ class _HierTrainStaged(torch.autograd.Function):
 
 @torch.library.custom_op("flexsae_amd::hier_train_sliced", mutates_args=())
 def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor,
-                      target: Tensor, need_dw: bool = True, hot: bool = False) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+                      target: Tensor, need_dw: bool = True, hot: bool = False,
+                      dense: bool = False) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     """Fused forward + reverse walk in column slices, each reduced right away (flat memory).
 
     Used when the contributions of a whole step do not fit the stage budget: the scratch is one
     slice of them (``set_hier_scratch_bytes``), and every slice gathers its weight-row pieces once
     for both walks.  Returns (loss, dvals, dbias, dW), the gradients for a unit upstream gradient;
     the backward scales them.  With ``need_dw`` false (a decoder whose weight takes no gradient)
-    the segment reductions are left out and the returned dW is empty."""
+    the segment reductions are left out and the returned dW is empty.  ``hot`` and ``dense`` are the
+    library's FLEXSAE_BWD_HOT_LATENTS and FLEXSAE_BWD_DENSE_LATENTS hints."""
     B, K, F, D = _validate(indices, weight, vals, bias, target)
     lib = _lib.load()
     indices, weight, vals, bias, target = (_prep(t) for t in (indices, weight, vals, bias, target))
@@ -690,7 +737,7 @@ def hier_train_sliced(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tenso
         if cached is not None:
             _pair_import(lib, shape, workspace, cached)
         flags = ((_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0) | (0 if need_dw else _lib.BWD_NO_DW) |
-                 hot_flag)
+                 hot_flag | (_lib.BWD_DENSE_LATENTS if dense else 0))
         rc = lib.flexsae_hier_fwd_bwd(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
                                       _ptr(target), _ptr(loss), _ptr(dW) if need_dw else None,
                                       _DTYPES[dw_dtype], _ptr(dvals),
@@ -711,7 +758,7 @@ def _unit_dw_dtype(weight_dtype):
 
 
 @hier_train_sliced.register_fake
-def _(indices, weight, vals, bias, target, need_dw=True, hot=False):
+def _(indices, weight, vals, bias, target, need_dw=True, hot=False, dense=False):
     dw_dtype = _unit_dw_dtype(weight.dtype)
     return (weight.new_empty((), dtype=torch.float32), vals.new_empty(vals.shape, dtype=torch.float32),
             weight.new_empty((weight.shape[1],), dtype=torch.float32),
@@ -748,6 +795,8 @@ def hier_sgd_step(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, t
         slice_cols = _hier_slice_cols(B, K, F, D, weight.dtype)
         # hot-latent accumulators: the same decision as the loss takes (set_hot_latents)
         hot_flag = _lib.BWD_HOT_LATENTS if _use_hot_latents(B, K, F, D, weight.dtype, dev, _is_traced(weight)) else 0
+        dense_flag = (_lib.BWD_DENSE_LATENTS
+                      if _use_dense_latents(B, K, F, D, weight.dtype, dev, _is_traced(weight)) else 0)
         if hot_flag:
             slice_cols = _hot_slice_cols(B, slice_cols, dev)
         ws_bytes = lib.flexsae_hier_fwd_bwd_workspace_bytes_flags(ctypes.byref(shape), slice_cols, hot_flag)
@@ -763,7 +812,8 @@ def hier_sgd_step(indices: Tensor, weight: Tensor, vals: Tensor, bias: Tensor, t
         rc = lib.flexsae_hier_sgd_step(ctypes.byref(shape), _ptr(indices), _ptr(weight), _ptr(vals), _ptr(bias),
                                        _ptr(target), _ptr(g), _ptr(loss), _ptr(dvals), _ptr(dbias),
                                        _ptr(workspace), ws_bytes,
-                                       (_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0) | hot_flag, _ptr(flag),
+                                       (_lib.BWD_REUSE_PAIR_LIST if cached is not None else 0) | hot_flag | dense_flag,
+                                       _ptr(flag),
                                        _stream())
         _lib.check(rc, "flexsae_hier_sgd_step")
         if cached is None:
@@ -861,9 +911,10 @@ def _is_traced(t: Tensor) -> bool:
 
 
 def _train_sliced_setup_context(ctx, inputs, output):
-    indices, weight, vals, bias, target, need_dw, hot = inputs
+    indices, weight, vals, bias, target, need_dw, hot, dense = inputs
     ctx.need_dw = need_dw
     ctx.hot = hot
+    ctx.dense = dense
     _, dvals, dbias, dW = output
     ctx.mark_non_differentiable(dvals, dbias, dW)
     ctx.leaf_dtypes = (vals.dtype, bias.dtype)
@@ -881,7 +932,7 @@ def _train_sliced_setup_context(ctx, inputs, output):
 
 def _train_sliced_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_dw):
     if grad_loss is None:
-        return None, None, None, None, None, None, None
+        return None, None, None, None, None, None, None, None
     if ctx.needs_input_grad[1] and not ctx.need_dw:
         raise RuntimeError("hier_train_sliced was called with need_dw=False but weight requires a gradient")
     g = grad_loss.to(torch.float32)
@@ -900,12 +951,12 @@ def _train_sliced_backward(ctx, grad_loss, grad_dvals, grad_dbias, grad_dw):
             if dW is None:
                 # a second backward through a retained graph: the buffer went with the first one
                 with torch.no_grad():
-                    _, dvals, dbias, dW = hier_train_sliced(indices, weight, vals, bias, target, True, ctx.hot)
+                    _, dvals, dbias, dW = hier_train_sliced(indices, weight, vals, bias, target, True, ctx.hot, ctx.dense)
             if dW.dtype == weight.dtype:
                 scale_(dW, g)
             else:  # fp16 weights: the fp32 unit gradient meets the upstream gradient before its only rounding
                 dW = scale_to(dW, g, weight.dtype)
-    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None, None, None
+    return None, dW, (dvals * g).to(vdt), (dbias * g).to(bdt), None, None, None, None
 
 
 hier_train_sliced.register_autograd(_train_sliced_backward, setup_context=_train_sliced_setup_context)
@@ -961,7 +1012,9 @@ def triton_hierarchical_sae_loss(indices: Tensor, weight: Tensor, vals: Tensor, 
             F, D = weight.shape
             hot = bool(weight.requires_grad) and _use_hot_latents(B, K, F, D, weight.dtype, weight.device,
                                                                    _is_traced(weight))
-            return hier_train_sliced(indices, weight, vals, bias, target, bool(weight.requires_grad), hot)[0]
+            dense = bool(weight.requires_grad) and _use_dense_latents(B, K, F, D, weight.dtype, weight.device,
+                                                                       _is_traced(weight))
+            return hier_train_sliced(indices, weight, vals, bias, target, bool(weight.requires_grad), hot, dense)[0]
     return hier_fwd(indices, weight, vals, bias, target)[0]
 
 

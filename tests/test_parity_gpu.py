@@ -720,6 +720,70 @@ def test_topk_residual_precision_switch():
     _check_against_oracle("topk", args, torch.bfloat16, 0.7, got, ref_tols=False)
 
 
+@pytest.mark.parametrize("zipf,dtype", [(None, torch.bfloat16), (1.1, torch.bfloat16), (None, torch.float32)])
+def test_dense_latents_hint_changes_no_bit(zipf, dtype):
+    """Shapes with at most two pairs per latent reduce from a list of the latents ordered by pair
+    count unless FLEXSAE_BWD_DENSE_LATENTS says most latents have pairs: the same results either way,
+    bit for bit (training step and fused SGD update), and flexsae_hier_pair_stats counts the latents
+    without pairs that the choice depends on."""
+    import ctypes
+    B, K, F, D = 256, 32, 5000, 384
+    assert B * K <= 2 * F
+    cpu_args = make_inputs(B, K, F, D, dtype=dtype, seed=37, zipf_s=zipf, unique=True)
+    idx, W, v, b, t = _to_dev(cpu_args)
+    DENSE = abi._lib.BWD_DENSE_LATENTS
+    outs = {}
+    for flags in (0, DENSE):
+        rc, loss, dW, dv, db, ws = abi.hier_train(idx, W, v, b, t, dw_dtype=dtype, slice_cols=128, flags=flags,
+                                                  keep_workspace=True)
+        assert rc == 0, abi._lib.status_string(rc)
+        outs[flags] = (loss, dW, dv, db)
+        stats = torch.zeros(3, dtype=torch.int32, device=DEV)
+        sh = abi.shape_of(idx, W, v, b.dtype, t.dtype)
+        assert abi._lib.load().flexsae_hier_pair_stats(ctypes.byref(sh), abi.ptr(ws), abi.ptr(stats), abi.stream()) == 0
+        counts = np.bincount(cpu_args[0].numpy().ravel(), minlength=F)
+        assert [int(x) for x in stats.cpu()][::2] == [int((counts > 64).sum()), int((counts == 0).sum())]
+    for a, c in zip(outs[0], outs[DENSE]):
+        assert torch.equal(a, c)
+    L, rW, rv, rb = oracle.loss_grads(oracle.HIER, *cpu_args)
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-4
+    assert rel_err(outs[DENSE][1].double().cpu(), rW) <= tol and rel_err(outs[DENSE][2].cpu(), rv) <= tol
+    # the in-place update
+    upd = {}
+    for flags in (0, DENSE):
+        Wn = W.clone()
+        rc, loss, dv, db = abi.hier_sgd_step(idx, Wn, v, b, t, 0.25, slice_cols=128, flags=flags)
+        assert rc == 0, abi._lib.status_string(rc)
+        upd[flags] = Wn
+    assert torch.equal(upd[0], upd[DENSE])
+
+
+def test_dense_latents_follow_the_previous_step():
+    """Through the package: a shape with two pairs per latent starts with the row-count list; uniform
+    indices (an eighth of the latents empty) drop it from the second step on, skewed ones keep it."""
+    flex.set_dense_latents("auto")
+    flex.set_hot_latents("off")  # (skewed indices would switch to the accumulators at the second step)
+    B, K, F, D = 512, 16, 4096, 256
+    try:
+        for zipf, want_dense in ((None, True), (1.1, False)):
+            cpu_args = make_inputs(B, K, F, D, dtype=torch.bfloat16, seed=38, zipf_s=zipf, unique=True)
+            idx, W, v, b, t = _to_dev(cpu_args)
+            flex.ops._hot_auto.clear()
+            grads = []
+            for step in range(3):
+                assert flex.ops._use_dense_latents(B, K, F, D, torch.bfloat16, W.device) == (want_dense and step > 0)
+                Wl = W.clone().requires_grad_()
+                flex.triton_hierarchical_sae_loss(idx, Wl, v, b, t).backward()
+                torch.cuda.synchronize()
+                grads.append(Wl.grad)
+            assert torch.equal(grads[0], grads[1]) and torch.equal(grads[1], grads[2])
+            L, rW, _, _ = oracle.loss_grads(oracle.HIER, *cpu_args)
+            assert rel_err(grads[2].double().cpu(), rW) <= 1e-2
+    finally:
+        flex.set_dense_latents(None)
+        flex.set_hot_latents(None)
+
+
 def test_topk_workspace_query_covers_both_residual_layouts():
     """bf16 weights, K = 512: the fp32-residual variant works on narrower tiles and needs more room
     for its per-tile shares of dvals than the bf16 one; the size query takes no flags and must
