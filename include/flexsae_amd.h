@@ -56,9 +56,10 @@ enum { FLEXSAE_FLAG_INDEX_RANGE = 1 };
 /* flags for the backward entry points */
 enum {
   FLEXSAE_BWD_OUTPUTS_PREZEROED = 1, /* caller already zero-filled the accumulators            */
-  /* flexsae_hier_bwd only: */
+  /* the hierarchical entry points that take a workspace: */
   FLEXSAE_BWD_REUSE_PAIR_LIST = 2,   /* the workspace still holds the pair list of a previous   */
                                      /* call with the same indices and shape: do not rebuild it */
+  /* flexsae_hier_bwd (and, for measurements, flexsae_hier_fwd_bwd): */
   FLEXSAE_BWD_SWEEP_ONLY = 4,        /* run only the sweep kernels (contributions stay in the   */
                                      /* workspace; meaningful when one slice covers all of D)   */
   FLEXSAE_BWD_REDUCE_ONLY = 8,       /* run only the segment reductions on the contributions    */
@@ -222,8 +223,8 @@ int flexsae_hier_bwd(const flexsae_shape *shape, const int64_t *indices, const v
  * 16-bit weights, 64 or 128 for fp32) when D is a multiple of the reduction's 16-byte lane width
  * (8 columns of bf16 contributions, 4 of fp32) -- the reduction then works on 256-byte pieces --
  * and to whole 256-column tiles otherwise; slice_cols <= 0 asks for the minimum; 0 is returned for
- * unsupported shapes.  Narrow slices keep one slice of contributions in the memory-side cache
- * between the kernel that writes it and the reduction that reads it.  A workspace from
+ * unsupported shapes.  A slice is reduced right after it has been written, while part of it may
+ * still be in the memory-side cache (256-column slices measured fastest at B*K = 2^19).  A workspace from
  * flexsae_hier_bwd_workspace_bytes is accepted as well.  The query assumes a dW aligned for that
  * 16-byte lane width (4 elements of fp32 or fp16 contributions' gradient, 8 of bf16); a dW aligned
  * less than that switches the piece reduction off, slices are then whole 256-column tiles, and a
@@ -286,7 +287,10 @@ int flexsae_hier_fwd_bwd(const flexsae_shape *shape, const int64_t *indices, con
  * staged contributions: D a multiple of 8 for bf16 weights (bf16 contributions, weight rows 16-byte
  * aligned), of 4 for fp32 and fp16 weights (fp32 contributions; weight rows aligned to 4 elements:
  * 16 bytes for fp32, 8 for fp16); otherwise FLEXSAE_ERR_UNSUPPORTED.  Workspace as for
- * flexsae_hier_fwd_bwd; the only flag accepted is FLEXSAE_BWD_REUSE_PAIR_LIST.
+ * flexsae_hier_fwd_bwd (for FLEXSAE_BWD_HOT_LATENTS from the _flags query); the flags accepted are
+ * FLEXSAE_BWD_REUSE_PAIR_LIST, FLEXSAE_BWD_HOT_LATENTS (the accumulators' sums update the weight rows
+ * of the hot latents the same way), FLEXSAE_BWD_REUSE_HOT_TABLES and FLEXSAE_BWD_DENSE_LATENTS; others
+ * are ignored.
  * replaces: the dense dW of the backward (hierarchical_kernels.py:241-243, 294-297) together with
  *           the optimizer pass that consumes it in a training loop written like reference
  *           example.py:76-77 with torch.optim.SGD (no momentum, no weight decay: for those the
