@@ -590,7 +590,7 @@ void launch_train_kernel_k(const flexsae_shape *s, const TrainArgs &ta, const in
 template <typename WT, typename PT>
 void launch_train_hot_kernel(const flexsae_shape *s, const TrainArgs &ta, const int64_t *indices,
                              const void *weight, const void *vals, float coef, const uint32_t *hslot, void *P,
-                             float *dvals, float *s_final, int d_pad, float *loss_partial, int *status_flag,
+                             float *dvals, float *colsum_part, float *loss_partial, int *status_flag,
                              int64_t cols, int col0, int slice_w, hipStream_t st, HotFinalize fin,
                              const HotBlockFinalize &hfin, uint32_t *ctrl, float *hot_partial,
                              int n_row_blocks, int headroom) {
@@ -609,7 +609,7 @@ void launch_train_hot_kernel(const flexsae_shape *s, const TrainArgs &ta, const 
                                    : (off32 ? hier_train_hot_kernel<WT, PT, KM, false, true>                    \
                                             : hier_train_hot_kernel<WT, PT, KM, false, false>);                 \
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kHotThreads), 0, st, indices, weight, vals, s->vals_dtype, ta.bias, \
-                       s->bias_dtype, ta.target, s->target_dtype, coef, hslot, P, dvals, s_final, d_pad,        \
+                       s->bias_dtype, ta.target, s->target_dtype, coef, hslot, P, dvals, colsum_part,           \
                        loss_partial, status_flag, s->B, n_tiles, n_row_blocks, col0, slice_w,                   \
                        static_cast<int>(s->K), s->F, static_cast<int>(s->D), ctrl, hot_partial, headroom, fin, hfin); \
   } while (0)
@@ -787,7 +787,7 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
     const int tps = static_cast<int>(cols / pl.tile);
     if (train && do_sweep && hot) {
       launch_train_hot_kernel<WT, PT>(s, *train, indices, weight, vals, coef,
-                                      reinterpret_cast<const uint32_t *>(ws + pl.off_hslot), P, dv_part, s_final, d_pad,
+                                      reinterpret_cast<const uint32_t *>(ws + pl.off_hslot), P, dv_part, colsum_part,
                                       reinterpret_cast<float *>(ws + pl.off_loss), status_flag, cols,
                                       static_cast<int>(col0), sw, st, pending, pending_hot, hot_ctrl,
                                       hot_partial[slice_no & 1], static_cast<int>(pl.n_row_blocks), hot_headroom);
@@ -850,7 +850,8 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
   // one launch: dvals = its per-tile shares added in tile order; stage 1 of dbias = column sums of
   // s_final over the rows, in a fixed order; the loss of the training step from its partials
   {
-    const unsigned n_colsum_blocks = static_cast<unsigned>(ceil_div(D, 256) * ceil_div(n_chunks, 4));
+    // (the hot-latent training step has formed stage 1 of the column sums on chip)
+    const unsigned n_colsum_blocks = hot ? 0u : static_cast<unsigned>(ceil_div(D, 256) * ceil_div(n_chunks, 4));
     const unsigned n_dvals_blocks = grid_for(s->B * s->K, 1024, 2048);
     hipLaunchKernelGGL(hier_epilogue_kernel, dim3(1 + n_colsum_blocks + n_dvals_blocks), dim3(1024), 0, st,
                        train ? reinterpret_cast<const float *>(ws + pl.off_loss) : static_cast<const float *>(nullptr),
@@ -859,8 +860,10 @@ void launch_hier_slices(const flexsae_shape *s, const HierBwdPlan &pl, int64_t s
                        static_cast<int64_t>(d_pad), D, colsum_part, n_colsum_blocks, dv_part,
                        static_cast<int>(d_used / (train ? train_tile_cols(s) : kWave * sweep_vec)), s->B * s->K, dvals);
   }
+  // (one partial per block of kHotRowsPerBlock rows from the hot-latent step, else per chunk of kColsumRows)
   hipLaunchKernelGGL(colsum_final_kernel, dim3(static_cast<unsigned>(ceil_div(D, 256))), dim3(256), 0, st,
-                     colsum_part, n_chunks, D, static_cast<const float *>(nullptr), 1.0f, dbias);
+                     colsum_part, hot ? static_cast<int>(pl.n_row_blocks) : n_chunks, D,
+                     static_cast<const float *>(nullptr), 1.0f, dbias);
 }
 
 template <typename WT, typename PT, int VEC>

@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
     const void *__restrict__ vals, int vals_dtype, const void *__restrict__ bias, int bias_dtype,
     const void *__restrict__ target, int target_dtype, float coef,
     const uint32_t *__restrict__ hslot, void *__restrict__ P, float *__restrict__ dv_part,
-    float *__restrict__ s_final, int s_final_ld, float *__restrict__ loss_partial,
+    float *__restrict__ colsum_part, float *__restrict__ loss_partial,
     int *status_flag, int64_t B, int n_tiles, int n_row_blocks, int col0, int slice_w, int K, int64_t F, int D,
     uint32_t *__restrict__ ctrl, float *__restrict__ hot_partial, int headroom, HotFinalize fin,
     HotBlockFinalize hfin) {
@@ -330,6 +330,7 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
   static_assert(sizeof(raw_t) == 4 && KMAX <= kWave && KMAX % 8 == 0, "16-bit weights, at most 64 steps");
   __shared__ int acc_lds[kHotMax * kHotCols];
   __shared__ int exp_lds[kHotWaves];
+  __shared__ float colsum_lds[kHotWaves][kHotCols];  // each wavefront's sum of S over its rows (for dbias)
   __shared__ int ask_lds;   // the largest exponent a deferred row asked for
   __shared__ int bad_lds;   // a row's bound was not finite
   const int lane = lane_id();
@@ -343,6 +344,7 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
   const int rb = static_cast<int>(blockIdx.x / static_cast<unsigned>(n_tiles));
   const int n_hot = static_cast<int>(ctrl[kHotNHot] < static_cast<uint32_t>(kHotMax) ? ctrl[kHotNHot] : kHotMax);
   for (int i = threadIdx.x; i < n_hot * kHotCols; i += kHotThreads) acc_lds[i] = 0;
+  for (int i = threadIdx.x; i < kHotWaves * kHotCols; i += kHotThreads) (&colsum_lds[0][0])[i] = 0.f;
   if (threadIdx.x == 0) {
     ask_lds = kHotExpMin - 1;
     bad_lds = 0;
@@ -550,11 +552,16 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
       }
       // this tile's share of dvals; the epilogue adds the tiles up in order
       if (lane < K) dv_part[(static_cast<int64_t>(col0 / kHotCols) + t) * (B * K) + pair0 + lane] = my_dval;
-      if (!active) {
+      // the row's final S (the gradient of its reconstruction) is only needed summed over the rows,
+      // for dbias: summed here per wavefront in row order, the wavefronts' sums added in order at
+      // the end of the block, the blocks' sums in order by colsum_final_kernel -- a fixed order that
+      // does not depend on the slice width (a deferred row is walked twice with the same S: counted
+      // in the first pass).  The plain step sums the same values in another fixed order (runs of 64
+      // rows), so dbias may differ from its in the last bits.
+      if (pass == 0) {
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) S[c] = 0.f;
+        for (int c = 0; c < VEC; ++c) colsum_lds[wv][lane * VEC + c] += S[c];
       }
-      store_vec<float, VEC>(s_final, b * s_final_ld + col0 + pc, S);
     }
     if (pass == 0) {
       // rows left for the second pass anywhere in the block: raise the block's exponent to the
@@ -583,6 +590,16 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
     const float unscale = bad_lds ? __builtin_nanf("") : __builtin_ldexpf(1.0f, exp_block - 22);
     float *dst = hot_partial + (static_cast<int64_t>(t) * n_row_blocks + rb) * (static_cast<int64_t>(kHotMax) * kHotCols);
     for (int j = threadIdx.x; j < n_hot * kHotCols; j += kHotThreads) dst[j] = static_cast<float>(acc_lds[j]) * unscale;
+  }
+  // stage 1 of dbias for this block's rows and columns: the wavefronts' sums in order
+  if (threadIdx.x < kHotCols) {
+    const int d = col0 + t * kHotCols + static_cast<int>(threadIdx.x);
+    if (d < D) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < kHotWaves; ++w2) sum += colsum_lds[w2][threadIdx.x];
+      colsum_part[static_cast<int64_t>(rb) * D + d] = sum;
+    }
   }
 }
 
