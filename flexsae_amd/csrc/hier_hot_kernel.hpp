@@ -439,6 +439,9 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
               __builtin_memcpy(&raw[k], &dw, sizeof(raw_t));
             }
           }
+          // all gathers are in flight before the walk waits for the first of them: left to itself
+          // the scheduler starts the walk's first step between the first two gathers
+          __builtin_amdgcn_sched_barrier(0);
         }
         // forward walk
         const int kb_fwd = k_bound();
@@ -550,8 +553,16 @@ __global__ __launch_bounds__(kHotThreads) void hier_train_hot_kernel(
           if ((lane >> 3) == (k8 >> 3)) my_dval = tot;
         }
       }
-      // this tile's share of dvals; the epilogue adds the tiles up in order
-      if (lane < K) dv_part[(static_cast<int64_t>(col0 / kHotCols) + t) * (B * K) + pair0 + lane] = my_dval;
+      // this tile's share of dvals; the epilogue adds the tiles up in order.  (A uniform base plus a
+      // lane number formed here: kept across the walks, the lane's 64-bit address is spilled, and
+      // its reload waits for every store of the row.)
+      {
+        uint32_t z = 0;
+        asm volatile("" : "+s"(z));  // a zero the optimiser cannot see through
+        const uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z));
+        float *const dv_row = dv_part + (static_cast<int64_t>(col0 / kHotCols) + t) * (B * K) + pair0;
+        if (ln < static_cast<uint32_t>(K)) dv_row[ln] = my_dval;
+      }
       // the row's final S (the gradient of its reconstruction) is only needed summed over the rows,
       // for dbias: summed here per wavefront in row order, the wavefronts' sums added in order at
       // the end of the block, the blocks' sums in order by colsum_final_kernel -- a fixed order that
